@@ -8,9 +8,10 @@ from .registry import (config_class_for, config_from_dict, config_from_dir,
 from .qwen3 import Qwen3Config
 from .bikovik import BikovikConfig
 from .biberax import BiberaxConfig
+from .toripel import ToripelConfig
 
 __all__ = [
     "ConfigError", "LayerSpec", "ModelConfig", "ModelSpec", "PartSpec", "ScheduleEntry",
     "config_class_for", "config_from_dict", "config_from_dir", "known_architectures",
-    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig", "BiberaxConfig",
+    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig", "BiberaxConfig", "ToripelConfig",
 ]

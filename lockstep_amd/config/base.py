@@ -115,6 +115,10 @@ class ModelSpec:
     head: PartSpec
     #: positions a request may use (its tokens are at positions 0 .. max_positions - 1); None: no bound
     max_positions: int | None = None
+    #: copies of a row that the residual stream holds (``[T, residual_copies * hidden_size]``): one, or the
+    #: several that an arrangement with hyper-connections reads and writes; the embedding fills them and the
+    #: final norm reads their sum
+    residual_copies: int = 1
 
     def cache_units(self) -> int:
         return 1 + max((e.cache for e in self.schedule), default=-1)

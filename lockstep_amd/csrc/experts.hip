@@ -5,7 +5,8 @@
 //   chosen(t)   = the `top` experts with the largest z[t] (the lower index wins a tie), in that order
 //   w[t, k]     = softmax over the chosen logits alone
 //   expert e    : y = act(W_gate[e] x, W_up[e] x),  out = W_down[e] y
-//                 act(g, u) = g' sigmoid(alpha g') (u' + 1),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
+//                 act(g, u) = g' sigmoid(alpha g') (u' + shift),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
+//                 (an infinite limit, alpha 1 and shift 0: the plain gated unit silu(g) u)
 //   P[k][t]     = w[t, k] * expert chosen(t)[k] (x[t])        (float; the caller adds the slices in order)
 //
 // (1) route: a wave a token picks the experts and their weights.  (2) group: the (token, choice) pairs
@@ -77,6 +78,17 @@ __device__ __forceinline__ void pick_top(const float* __restrict__ row, const fl
     picked[lane] = my_pick;
     share[lane] = ex / sum;
   }
+}
+
+// The experts of a token come from a table instead of a router: row token_id of table [vocab][top] names them (its
+// entries differ), and every one weighs 1 / top.
+__global__ __launch_bounds__(256) void route_table_kernel(const int* __restrict__ token_ids, const int* __restrict__ table,
+                                                          int n_tokens, int top, int* __restrict__ expert,
+                                                          float* __restrict__ weight) {
+  const long pair = (long)blockIdx.x * 256 + threadIdx.x;
+  if (pair >= (long)n_tokens * top) return;
+  expert[pair] = table[(long)token_ids[pair / top] * top + pair % top];
+  weight[pair] = 1.0f / (float)top;
 }
 
 __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ z, long ldz,
@@ -167,13 +179,22 @@ __global__ __launch_bounds__(1024) void route_small_kernel(const float* __restri
                                                            const float* __restrict__ bias, int n_tokens, int E, int top,
                                                            int rows_a_tile, int* __restrict__ expert,
                                                            float* __restrict__ weight, int* __restrict__ order,
-                                                           int* __restrict__ tiles, int cap) {
+                                                           int* __restrict__ tiles, int cap,
+                                                           const int* __restrict__ token_ids, const int* __restrict__ table) {
   __shared__ int picks_s[kSmallPairs];
   __shared__ float share_s[16][kMaxTop];
   __shared__ int counts_s[kSmallExperts];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int P = n_tokens * top;
-  for (int t = w; t < n_tokens; t += 16) {
+  if (table) {   // the picks are looked up, not chosen
+    for (int pair = threadIdx.x; pair < P; pair += 1024) {
+      const int e = table[(long)token_ids[pair / top] * top + pair % top];
+      picks_s[pair] = e;
+      expert[pair] = e;
+      weight[pair] = 1.0f / (float)top;
+    }
+  }
+  for (int t = w; t < n_tokens && !table; t += 16) {
     pick_top(z + (long)t * ldz, bias, E, top, lane, picks_s + t * top, share_s[w]);
     if (lane < top) {
       expert[(long)t * top + lane] = picks_s[t * top + lane];
@@ -197,7 +218,7 @@ template <typename T, int RT, int KS>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ x, long ldx,
                                                               const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                               int F, int K, int top, const int* __restrict__ order,
-                                                              const int* __restrict__ tiles, float limit, float alpha,
+                                                              const int* __restrict__ tiles, float limit, float alpha, float shift,
                                                               T* __restrict__ act, long ldy) {
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
   const int e = tiles[4 * blockIdx.x];
@@ -275,7 +296,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
       if (c < F) {
         const float g = fminf(acc_g[r][i], limit);
         const float u = fminf(fmaxf(acc_u[r][i], -limit), limit);
-        dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + 1.0f));
+        dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + shift));
       }
     }
   }
@@ -442,7 +463,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_tiled_kernel(const T* __r
                                                                     const T* __restrict__ w_up, int F, int K, int top,
                                                                     const int* __restrict__ order,
                                                                     const int* __restrict__ tiles, float limit, float alpha,
-                                                                    T* __restrict__ act, long ldy) {
+                                                                    float shift, T* __restrict__ act, long ldy) {
   __shared__ __attribute__((aligned(16))) char lds[2 * 3 * 64 * kLdsRow];
   const int e = tiles[4 * blockIdx.x];
   if (e < 0) return;
@@ -474,7 +495,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_tiled_kernel(const T* __r
         if (c < F) {
           const float g = fminf(product.acc[0][rt][ct][i], limit);
           const float u = fminf(fmaxf(product.acc[1][rt][ct][i], -limit), limit);
-          dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + 1.0f));
+          dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + shift));
         }
       }
   }
@@ -549,7 +570,7 @@ extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int
   const int P = n_tokens * top;
   if (P <= kSmallPairs && E <= kSmallExperts) {
     hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(1024), 0, s, z, ldz, bias, n_tokens, E, top, rows_a_tile,
-                       expert, weight, order, tiles, cap);
+                       expert, weight, order, tiles, cap, (const int*)nullptr, (const int*)nullptr);
   } else {
     hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, s, z, ldz, bias, n_tokens, E, top,
                        expert, weight);
@@ -559,12 +580,34 @@ extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int
   return check_launch("experts_route");
 }
 
+// The same grouping for experts that a table names: token_ids [n_tokens], table [vocab][top] with entries in [0, E).
+extern "C" int ls_experts_route_table(const int* token_ids, const int* table, int n_tokens, int E, int top,
+                                      int rows_a_tile, int* expert, float* weight, int* order, int* tiles, int cap,
+                                      int* counts, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && top <= E, "experts_route_table: %d tokens, %d experts, %d a token", n_tokens, E, top);
+  LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_route_table: tiles of %d rows", rows_a_tile);
+  LS_REQUIRE(token_ids && table && expert && weight && order && tiles && counts, "experts_route_table: null operand");
+  LS_REQUIRE(cap >= ls_experts_tile_capacity(n_tokens, E, top, rows_a_tile), "experts_route_table: %d tiles are too few", cap);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int P = n_tokens * top;
+  if (P <= kSmallPairs && E <= kSmallExperts) {
+    hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(1024), 0, s, (const float*)nullptr, 0L, (const float*)nullptr,
+                       n_tokens, E, top, rows_a_tile, expert, weight, order, tiles, cap, token_ids, table);
+  } else {
+    hipLaunchKernelGGL(route_table_kernel, dim3((P + 255) / 256), dim3(256), 0, s, token_ids, table, n_tokens, top, expert,
+                       weight);
+    hipLaunchKernelGGL(route_count_kernel, dim3(E), dim3(64), 0, s, expert, P, counts);
+    hipLaunchKernelGGL(route_place_kernel, dim3(E), dim3(64), 0, s, expert, counts, P, E, rows_a_tile, order, tiles, cap);
+  }
+  return check_launch("experts_route_table");
+}
+
 // x [n_tokens][ldx]; w_gate, w_up [E][F][K]; w_down [E][N][F]; act: scratch [n_tokens * top][ldy] of the compute
 // dtype; P [top][n_tokens][N] float.
 extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* w_gate, const void* w_up,
                                 const void* w_down, int n_tokens, int E, int top, int K, int F, int N,
                                 int rows_a_tile, const int* order, const int* tiles, int cap, const float* weight,
-                                float limit, float alpha, void* act, long ldy, float* P, void* stream) {
+                                float limit, float alpha, float shift, void* act, long ldy, float* P, void* stream) {
   LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && K > 0 && F > 0 && N > 0 && ldx >= K && ldy >= F, "experts_apply: bad sizes");
   LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_apply: tiles of %d rows", rows_a_tile);
   LS_REQUIRE(x && w_gate && w_up && w_down && order && tiles && weight && act && P && cap > 0, "experts_apply: null operand");
@@ -582,7 +625,7 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
 #define LS_EXPERTS(T_, RT_, KS_)                                                                                      \
   do {                                                                                                                \
     hipLaunchKernelGGL((experts_gate_up_kernel<T_, RT_, KS_>), grid_up, dim3(256), 0, s, (const T_*)x, ldx,           \
-                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, (T_*)act, ldy);     \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, (T_*)act, ldy);     \
     hipLaunchKernelGGL((experts_down_kernel<T_, RT_, KS_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,          \
                        (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
   } while (0)
@@ -591,7 +634,7 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
 #define LS_EXPERTS_STAGED(T_)                                                                                         \
   do {                                                                                                                \
     hipLaunchKernelGGL(experts_gate_up_tiled_kernel<T_>, grid_up, dim3(256), 0, s, (const T_*)x, ldx,                 \
-                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, (T_*)act, ldy);     \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, (T_*)act, ldy);     \
     hipLaunchKernelGGL(experts_down_tiled_kernel<T_>, grid_down, dim3(256), 0, s, (const T_*)act, ldy,                \
                        (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
   } while (0)

@@ -1,0 +1,582 @@
+// More kernels of the mixers library: a residual stream of several copies that every sublayer reads
+// as one weighted sum and writes back through a small mixing matrix (with the norm of the next reader
+// fused in), the passes around attention over a cached latent (norms of the latents, rotation of the
+// shared key part, queries brought into the latent's space by a product a head), and the gated delta
+// rule with its short convolutions.
+//
+// Everything here is computed in float whatever the compute dtype T is: T is the type of what a
+// matrix product reads next (and of the cache).  Per-row reductions have an order fixed by the row's
+// sizes alone; the recurrence walks a request's tokens in order, so nothing depends on how the
+// request was cut into steps or on what else is in the batch.
+
+#include "common.h"
+#include "mixers_api.h"
+
+namespace ls {
+
+struct SeqMeta {  // one per sequence of the step (all int32), as the step's upload lays it out
+  int q_off;      // first packed row
+  int q_len;      // rows in this step
+  int q_start;    // absolute position of the first row
+  int kv_len;     // q_start + q_len
+  int table_row;  // row of the block table, and the request's state slot
+  int reserved[3];
+};
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+
+// The four wave sums of a workgroup of 256 threads added in wave order; every thread gets the total.
+__device__ __forceinline__ float block_sum4(float v, float* scratch) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[w] = v;
+  __syncthreads();
+  return ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
+}
+
+// ---------------------------------------------------------------------------
+// A residual stream of n copies X [rows][n][W] (float).  One launch does, for a row, either or both of
+//   write:  y = P[0][row] + P[1][row] + ... (slices ascending, from +0: the sublayer's output, left as slice sums);
+//           X'_t = sum_s mix[s][t] X_s + gain[t] y      for all t at once from the old copies
+//   read:   u = sum_t take[t] X'_t   (take == null: the plain sum of the copies)
+//           out = u / sqrt(mean(u^2) + eps) * weight     (T)
+// Thread t of 256 owns the elements 1024 c + 4 t + {0..3}; the sum of squares adds them in ascending order, then
+// a butterfly over the wave and the wave sums in wave order.  `row` = rows[r] when a row list is given.
+// ---------------------------------------------------------------------------
+constexpr int kMaxStreams = 8;
+constexpr int kStreamChunks = 8;  // a row of up to 1024 * kStreamChunks elements keeps its u in registers
+
+template <typename T>
+__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X, long ldx, int n, int W,
+                                                           const float* __restrict__ P, int slices, long p_stride,
+                                                           const float* __restrict__ mix, const float* __restrict__ gain,
+                                                           const float* __restrict__ take, const float* __restrict__ weight,
+                                                           float eps, T* __restrict__ out, long ld_out,
+                                                           const int* __restrict__ rows) {
+  __shared__ float mix_s[kMaxStreams * kMaxStreams], gain_s[kMaxStreams], take_s[kMaxStreams], scratch[4];
+  const int r_out = blockIdx.x;
+  const long row = rows ? rows[r_out] : r_out;
+  if (threadIdx.x < n * n) mix_s[threadIdx.x] = P ? mix[threadIdx.x] : 0.f;
+  if (threadIdx.x < n) {
+    gain_s[threadIdx.x] = P ? gain[threadIdx.x] : 0.f;
+    take_s[threadIdx.x] = take ? take[threadIdx.x] : 1.0f;
+  }
+  __syncthreads();
+  float* x = X + row * ldx;
+  float u[kStreamChunks][4];
+  float part = 0.f;
+#pragma unroll
+  for (int c = 0; c < kStreamChunks; ++c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = 1024 * c + 4 * (int)threadIdx.x + i;
+      u[c][i] = 0.f;
+      if (e >= W) continue;
+      float copy[kMaxStreams];
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s) copy[s] = s < n ? x[(long)s * W + e] : 0.f;
+      if (P) {
+        const float* p = P + row * W + e;
+        float y = 0.f;
+        for (int s = 0; s < slices; ++s) y = y + p[s * p_stride];
+        float fresh[kMaxStreams];
+#pragma unroll
+        for (int t = 0; t < kMaxStreams; ++t) {
+          float v = 0.f;
+#pragma unroll
+          for (int s = 0; s < kMaxStreams; ++s)
+            if (s < n && t < n) v = v + mix_s[s * n + t] * copy[s];
+          fresh[t] = t < n ? v + gain_s[t] * y : 0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < kMaxStreams; ++t) {
+          copy[t] = fresh[t];
+          if (t < n) x[(long)t * W + e] = fresh[t];
+        }
+      }
+      float sum = 0.f;
+#pragma unroll
+      for (int t = 0; t < kMaxStreams; ++t)
+        if (t < n) sum = sum + take_s[t] * copy[t];
+      u[c][i] = sum;
+      part = part + sum * sum;
+    }
+  }
+  if (!out) return;
+  const float scale = 1.0f / sqrtf(block_sum4(part, scratch) / (float)W + eps);
+#pragma unroll
+  for (int c = 0; c < kStreamChunks; ++c) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = 1024 * c + 4 * (int)threadIdx.x + i;
+      if (e < W) out[(long)r_out * ld_out + e] = from_f32<T>((u[c][i] * scale) * weight[e]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Post pass of the down projections of attention over a latent: raw [T][ld] float = a (QR) | c (CR) | r (RD), the
+// last two absent for a layer that reads another layer's latent (has_kv == 0).
+//   a -> a / sqrt(mean(a^2) + eps) * a_weight            -> a_out [T][QR] (T)
+//   c -> c / sqrt(mean(c^2) + eps) * c_weight            -> key pages [page][0][slot][0 .. CR) and value pages
+//                                                           [page][0][0 .. CR)[slot]: the latent is key and value
+//   r -> rotated in neighbouring pairs (2i, 2i + 1) on its first `rot` dimensions at the token's position
+//                                                        -> key pages [page][0][slot][CR .. CR + RD), zeros up to Dp
+// One workgroup a token; the sums of squares as in streams_step_kernel.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void latent_post_kernel(
+    const float* __restrict__ raw, long ld, int QR, int CR, int RD, int Dp, int has_kv, const float* __restrict__ a_weight,
+    const float* __restrict__ c_weight, float eps, const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    int rot, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
+    const int* __restrict__ table, int table_stride, T* __restrict__ a_out, long lda, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int page_size) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* row = raw + (long)t * ld;
+  {
+    const float part = row_sumsq_part(row, QR, threadIdx.x, false);
+    const float scale = 1.0f / sqrtf(block_sum4(part, scratch) / (float)QR + eps);
+    for (int e = threadIdx.x; e < QR; e += 256) a_out[(long)t * lda + e] = from_f32<T>((row[e] * scale) * a_weight[e]);
+  }
+  if (!has_kv) return;
+  const int pos = tok_pos[t];
+  const int page = table[(long)seqs[tok_seq[t]].table_row * table_stride + pos / page_size];
+  const int slot = pos % page_size;
+  const float part = row_sumsq_part(row + QR, CR, threadIdx.x, false);
+  const float scale = 1.0f / sqrtf(block_sum4(part, scratch) / (float)CR + eps);
+  if (page < 0) return;
+  T* key = k_pages + ((long)page * page_size + slot) * Dp;
+  T* value = v_pages + (long)page * CR * page_size + slot;
+  for (int e = threadIdx.x; e < CR; e += 256) {
+    const T c = from_f32<T>((row[QR + e] * scale) * c_weight[e]);
+    key[e] = c;
+    value[(long)e * page_size] = c;
+  }
+  const float* r = row + QR + CR;
+  const int half = rot >> 1;
+  for (int i = threadIdx.x; i < Dp - CR; i += 256) {
+    float v = 0.f;
+    if (i < RD) {
+      v = r[i];
+      if (i < rot) {
+        const float other = r[i ^ 1], c = cos_table[(long)pos * half + (i >> 1)], s = sin_table[(long)pos * half + (i >> 1)];
+        v = (i & 1) ? v * c + other * s : v * c - other * s;
+      }
+    }
+    key[CR + i] = from_f32<T>(v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Post pass of the up projection of the queries: qf [T][ld] float holds, head by head, D plain dimensions and RD
+// rotated ones.  The plain ones go to plain_out [T][H*D] (T), the operand of the product that brings them into the
+// latent's space; the rotated ones are rotated (neighbouring pairs, first `rot` dimensions) and written where the
+// attention kernel reads them, behind the CR latent dimensions of a query head of Dp elements (zeros up to Dp).
+// One thread an element.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void latent_query_kernel(const float* __restrict__ qf, long ld, int n_tokens, int H, int D,
+                                                           int RD, int CR, int Dp, const float* __restrict__ cos_table,
+                                                           const float* __restrict__ sin_table, int rot,
+                                                           const int* __restrict__ tok_pos, T* __restrict__ plain_out,
+                                                           long ldp, T* __restrict__ q_out, long ldq) {
+  const int tail = Dp - CR, each = D + tail;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)n_tokens * H * each) return;
+  const int i = (int)(idx % each), head = (int)((idx / each) % H), t = (int)(idx / ((long)each * H));
+  const float* src = qf + (long)t * ld + (long)head * (D + RD);
+  if (i < D) {
+    plain_out[(long)t * ldp + head * D + i] = from_f32<T>(src[i]);
+    return;
+  }
+  const int j = i - D;
+  float v = 0.f;
+  if (j < RD) {
+    v = src[D + j];
+    if (j < rot) {
+      const int half = rot >> 1;
+      const long pos = tok_pos[t];
+      const float other = src[D + (j ^ 1)], c = cos_table[pos * half + (j >> 1)], s = sin_table[pos * half + (j >> 1)];
+      v = (j & 1) ? v * c + other * s : v * c - other * s;
+    }
+  }
+  q_out[(long)t * ldq + (long)head * Dp + CR + j] = from_f32<T>(v);
+}
+
+// ---------------------------------------------------------------------------
+// A product a head: out[t][head * o_stride + n] = sum_k w[head][n][k] x[t][head * x_stride + k], w [H][N][K].
+// A workgroup: 16 * RT rows of one head, four waves with 16 columns each.  The 16x16 MFMA atom with the weight rows
+// as first operand; a row's contraction is one chain over ascending K from zero.
+// ---------------------------------------------------------------------------
+template <typename T, int RT>
+__global__ __launch_bounds__(256) void heads_product_kernel(const T* __restrict__ x, long ldx, int x_stride,
+                                                            const T* __restrict__ w, int N, int K, int n_rows,
+                                                            T* __restrict__ out, long ldo, int o_stride, int x_aligned) {
+  constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
+  const int head = blockIdx.y;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int l16 = lane & 15, quad = lane >> 4;
+  const int col0 = (blockIdx.z * 4 + wv) * 16;
+  if (col0 >= N) return;
+  const bool w_ok = col0 + l16 < N;
+  const T* w_row = w + ((long)head * N + (w_ok ? col0 + l16 : 0)) * K;
+  const int row0 = blockIdx.x * 16 * RT;
+  const T* x_row[RT];
+  bool x_ok[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    x_ok[r] = row0 + 16 * r + l16 < n_rows;
+    x_row[r] = x + (long)(x_ok[r] ? row0 + 16 * r + l16 : 0) * ldx + (long)head * x_stride;
+  }
+  f32x4 acc[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool w_aligned = K % VEC == 0;
+  constexpr int U = 4;
+  for (int k0 = 0; k0 < K; k0 += U * KC) {
+    typename Atom<T>::vec_t a[U], b[U][RT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * KC + VEC * quad;
+      a[u] = load_vec<T>(w_row, 0, k, K, 0, w_ok, w_aligned);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) b[u][r] = load_vec<T>(x_row[r], 0, k, K, 0, x_ok[r], x_aligned != 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) Atom<T>::mma(acc[r], a[u], b[u][r]);
+  }
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (!x_ok[r]) continue;
+    T* dst = out + (long)(row0 + 16 * r + l16) * ldo + (long)head * o_stride;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = col0 + 4 * quad + i;
+      if (c < N) dst[c] = from_f32<T>(acc[r][i]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The gated delta rule.  raw [T][ld] float holds the projections q (G heads of D) | k (G of D) | v (H of DV) |
+// b (H) | a (H) | whatever follows.  Per request a state of floats: S [H][D][DV], then the last M - 1 inputs of the
+// short convolutions [M - 1][C], C = 2 G D + H DV channels, oldest first, zeros before the start.
+//
+// (1) delta_prep: a wave a (token, unit).  Units: the G query heads, the G key heads, the H value heads, and one for
+//     the gates.  A channel's convolution y = sum_m taps[c][m] in(p - (M - 1) + m) (m ascending) takes the inputs of
+//     this step from raw and those before it from the state; then silu; queries and keys become unit vectors
+//     x / sqrt(sum x^2 + unit_eps) (lane i adds the squares of the elements i, i + 64, ... ascending, then a
+//     butterfly), the query also times D^(-1/2).  Gates of head h: beta = sigmoid(b_h),
+//     decay = exp(-exp(A_log_h) softplus(a_h + dt_bias_h)).
+//     qk [T][2 G][dp] (queries, then keys; zeros beyond D), vv [T][H * DV], gates [T][H][2].
+// (2) delta_rule: a wave a (request, head, 16 columns of the state); lane (column lane / 4, quarter lane % 4)
+//     keeps the rows quarter * R + {0 .. R-1} of its column.  Per token, in order:
+//       kS = decay * sum_r S[r] k[r];  u = beta (v - kS);  S[r] = decay S[r] + k[r] u;  o = sum_r S[r] q[r]
+//     (the sums: a lane's rows ascending by fused multiply-adds, then the quarters by exchanges inside the quad; the
+//     decay multiplies the sum of the old state with the key, which is the decayed state's sum up to rounding).
+//     The operands of the next token are requested before a token is worked on.
+// (3) delta_conv_state: the last M - 1 inputs of every channel become the state of the next step.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void delta_prep_kernel(
+    const float* __restrict__ raw, long ld, int n_tokens, int G, int H, int D, int DV, int dp, int M,
+    const float* __restrict__ taps, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
+    const float* __restrict__ state, long state_stride, long conv_at, float* __restrict__ qk, float* __restrict__ vv,
+    float* __restrict__ gates) {
+  const int units = 2 * G + H + 1;
+  const long id = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (id >= (long)n_tokens * units) return;
+  const int t = (int)(id / units), unit = (int)(id % units), lane = threadIdx.x & 63;
+  const float* row = raw + (long)t * ld;
+  const int C = 2 * G * D + H * DV;
+  if (unit == units - 1) {
+    for (int h = lane; h < H; h += 64) {
+      gates[((long)t * H + h) * 2] = sigmoid_f(row[C + h]);
+      gates[((long)t * H + h) * 2 + 1] = expf(-expf(a_log[h]) * softplus_f(row[C + H + h] + dt_bias[h]));
+    }
+    return;
+  }
+  const SeqMeta m = seqs[tok_seq[t]];
+  const int pos = tok_pos[t];
+  const float* old = state + (long)m.table_row * state_stride + conv_at;
+  const bool is_v = unit >= 2 * G;
+  const int size = is_v ? DV : D;
+  const int c0 = is_v ? 2 * G * D + (unit - 2 * G) * DV : unit * D;
+  // channel c at this token: convolution over the last M inputs, then silu
+  auto channel = [&](int c) LS_INLINED {
+    float y = 0.f;
+    for (int a = 0; a < M; ++a) {
+      const int p = pos - (M - 1) + a;
+      const float in = p >= m.q_start ? raw[(long)(m.q_off + p - m.q_start) * ld + c]
+                                      : old[(long)(p - m.q_start + M - 1) * C + c];
+      y = y + taps[(long)c * M + a] * in;
+    }
+    return silu_f(y);
+  };
+  if (is_v) {
+    for (int i = lane; i < size; i += 64) vv[(long)t * H * DV + (c0 - 2 * G * D) + i] = channel(c0 + i);
+    return;
+  }
+  float part = 0.f;
+  for (int i = lane; i < size; i += 64) {
+    const float x = channel(c0 + i);
+    part = part + x * x;
+  }
+  float scale = 1.0f / sqrtf(wave_sum(part) + unit_eps);
+  if (unit < G) scale = scale * (1.0f / sqrtf((float)D));
+  float* dst = qk + ((long)t * 2 * G + unit) * dp;
+  for (int i = lane; i < dp; i += 64) dst[i] = i < size ? channel(c0 + i) * scale : 0.f;
+}
+
+__device__ __forceinline__ float quad4_sum(float v) {
+  v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes 1 0 3 2
+  v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));  // lanes 2 3 0 1
+  return v;
+}
+
+template <int R>
+__global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict__ qk, const float* __restrict__ vv,
+                                                        const float* __restrict__ gates, int G, int H, int D, int DV,
+                                                        const SeqMeta* __restrict__ seqs, float* __restrict__ state,
+                                                        long state_stride, float* __restrict__ out, long ldo) {
+  constexpr int dp = 4 * R;
+  const int seq = blockIdx.x / H, head = blockIdx.x % H;
+  const SeqMeta m = seqs[seq];
+  if (m.q_len <= 0) return;
+  const int lane = threadIdx.x, l16 = lane >> 2, quarter = lane & 3;
+  const int col = blockIdx.y * 16 + l16;
+  const bool col_ok = col < DV;
+  const int row0 = quarter * R;
+  const int kh = head / (H / G);
+  float* mine = state + (long)m.table_row * state_stride + (long)head * D * DV;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) S[r] = (row0 + r < D && col_ok) ? mine[(long)(row0 + r) * DV + col] : 0.f;
+  struct Operands {
+    f32x4 q[R / 4], k[R / 4];
+    float v, beta, decay;
+  };
+  auto fetch = [&](int t) LS_INLINED {
+    Operands x;
+    const float* q = qk + ((long)t * 2 * G + kh) * dp + row0;
+    const float* k = qk + ((long)t * 2 * G + G + kh) * dp + row0;
+#pragma unroll
+    for (int j = 0; j < R / 4; ++j) {
+      x.q[j] = *reinterpret_cast<const f32x4*>(q + 4 * j);
+      x.k[j] = *reinterpret_cast<const f32x4*>(k + 4 * j);
+    }
+    x.v = col_ok ? vv[(long)t * H * DV + head * DV + col] : 0.f;
+    x.beta = gates[((long)t * H + head) * 2];
+    x.decay = gates[((long)t * H + head) * 2 + 1];
+    return x;
+  };
+  Operands next = fetch(m.q_off);
+  for (int i = 0; i < m.q_len; ++i) {
+    const Operands now = next;
+    if (i + 1 < m.q_len) next = fetch(m.q_off + i + 1);
+    float ks = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) ks = fmaf(S[r], now.k[r >> 2][r & 3], ks);
+    ks = quad4_sum(ks) * now.decay;
+    const float u = now.beta * (now.v - ks);
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      S[r] = fmaf(now.k[r >> 2][r & 3], u, now.decay * S[r]);
+      o = fmaf(S[r], now.q[r >> 2][r & 3], o);
+    }
+    o = quad4_sum(o);
+    if (quarter == 0 && col_ok) out[(long)(m.q_off + i) * ldo + head * DV + col] = o;
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (row0 + r < D && col_ok) mine[(long)(row0 + r) * DV + col] = S[r];
+}
+
+__global__ __launch_bounds__(256) void delta_conv_state_kernel(const float* __restrict__ raw, long ld, int C, int M,
+                                                               const SeqMeta* __restrict__ seqs, float* __restrict__ state,
+                                                               long state_stride, long conv_at) {
+  const SeqMeta m = seqs[blockIdx.x];
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (m.q_len <= 0 || c >= C) return;
+  float* kept = state + (long)m.table_row * state_stride + conv_at;
+  // place a holds the input at position kv_len - (M - 1) + a: one of this step's, or one the state already holds
+  // further on (read before the ascending walk overwrites it)
+  for (int a = 0; a < M - 1; ++a) {
+    const int p = m.kv_len - (M - 1) + a;
+    kept[(long)a * C + c] = p >= m.q_start ? raw[(long)(m.q_off + p - m.q_start) * ld + c]
+                                           : kept[(long)(p - m.q_start + M - 1) * C + c];
+  }
+}
+
+}  // namespace ls
+
+using namespace ls;
+
+extern "C" int ls_streams_max() { return kMaxStreams; }
+extern "C" int ls_streams_max_width() { return 1024 * kStreamChunks; }
+
+extern "C" int ls_streams_step(int dtype, float* X, long ldx, int n, int width, const float* P, int slices, int p_rows,
+                               const float* mix, const float* gain, const float* take, const float* weight, float eps,
+                               void* out, long ld_out, const int* rows, int n_rows, void* stream) {
+  LS_REQUIRE(n_rows > 0 && n > 0 && n <= kMaxStreams && width > 0 && width <= 1024 * kStreamChunks && ldx >= (long)n * width,
+             "streams_step: %d copies of %d elements (at most %d of %d)", n, width, kMaxStreams, 1024 * kStreamChunks);
+  LS_REQUIRE(X && (P || out), "streams_step: nothing to do");
+  LS_REQUIRE(!P || (slices > 0 && p_rows > 0 && mix && gain), "streams_step: a write needs slices, mix and gain");
+  LS_REQUIRE(!out || (weight && ld_out >= width && eps > 0.f), "streams_step: a read needs a weight and eps");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long p_stride = (long)p_rows * width;
+#define LS_STREAMS(T_)                                                                                               \
+  hipLaunchKernelGGL(streams_step_kernel<T_>, dim3(n_rows), dim3(256), 0, s, X, ldx, n, width, P, slices, p_stride, \
+                     mix, gain, take, weight, eps, (T_*)out, ld_out, rows)
+  if (dtype == kF32)
+    LS_STREAMS(float);
+  else if (dtype == kBF16)
+    LS_STREAMS(bf16_t);
+  else
+    return fail("streams_step: unknown dtype %d", dtype);
+#undef LS_STREAMS
+  return check_launch("streams_step");
+}
+
+extern "C" int ls_latent_post(int dtype, const float* raw, long ld, int n_tokens, int QR, int CR, int RD, int Dp,
+                              int has_kv, const float* a_weight, const float* c_weight, float eps, const float* cos_table,
+                              const float* sin_table, int rot, int table_positions, int max_pos, const int* tok_seq,
+                              const int* tok_pos, const void* seqs, const int* table, int table_stride, void* a_out,
+                              long lda, void* k_pages, void* v_pages, int page_size, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && QR > 0 && raw && a_out && a_weight && lda >= QR && eps > 0.f, "latent_post: bad query latent");
+  LS_REQUIRE(ld >= QR + (has_kv ? CR + RD : 0), "latent_post: rows of %ld floats are too short", ld);
+  if (has_kv) {
+    LS_REQUIRE(CR > 0 && RD >= 0 && Dp >= CR + RD && c_weight && k_pages && v_pages && table && seqs && tok_seq && tok_pos &&
+                   page_size > 0 && table_stride > 0,
+               "latent_post: bad key/value latent");
+    LS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= RD, "latent_post: %d rotated dimensions of %d", rot, RD);
+    LS_REQUIRE(rot == 0 || (cos_table && sin_table && max_pos < table_positions),
+               "latent_post: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
+    LS_REQUIRE(max_pos / page_size < table_stride, "latent_post: position %d is beyond the block table", max_pos);
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define LS_LATENT_POST(T_)                                                                                            \
+  hipLaunchKernelGGL(latent_post_kernel<T_>, dim3(n_tokens), dim3(256), 0, s, raw, ld, QR, CR, RD, Dp, has_kv, a_weight, \
+                     c_weight, eps, cos_table, sin_table, rot, tok_seq, tok_pos, (const SeqMeta*)seqs, table,         \
+                     table_stride, (T_*)a_out, lda, (T_*)k_pages, (T_*)v_pages, page_size)
+  if (dtype == kF32)
+    LS_LATENT_POST(float);
+  else if (dtype == kBF16)
+    LS_LATENT_POST(bf16_t);
+  else
+    return fail("latent_post: unknown dtype %d", dtype);
+#undef LS_LATENT_POST
+  return check_launch("latent_post");
+}
+
+extern "C" int ls_latent_query(int dtype, const float* qf, long ld, int n_tokens, int H, int D, int RD, int CR, int Dp,
+                               const float* cos_table, const float* sin_table, int rot, int table_positions, int max_pos,
+                               const int* tok_pos, void* plain_out, long ldp, void* q_out, long ldq, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && H > 0 && D > 0 && RD >= 0 && CR > 0 && Dp >= CR + RD, "latent_query: bad sizes");
+  LS_REQUIRE(qf && plain_out && q_out && tok_pos && ld >= (long)H * (D + RD) && ldp >= (long)H * D && ldq >= (long)H * Dp,
+             "latent_query: bad operands");
+  LS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= RD, "latent_query: %d rotated dimensions of %d", rot, RD);
+  LS_REQUIRE(rot == 0 || (cos_table && sin_table && max_pos < table_positions),
+             "latent_query: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const long total = (long)n_tokens * H * (D + Dp - CR);
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+#define LS_LATENT_QUERY(T_)                                                                                          \
+  hipLaunchKernelGGL(latent_query_kernel<T_>, dim3(blocks), dim3(256), 0, s, qf, ld, n_tokens, H, D, RD, CR, Dp,     \
+                     cos_table, sin_table, rot, tok_pos, (T_*)plain_out, ldp, (T_*)q_out, ldq)
+  if (dtype == kF32)
+    LS_LATENT_QUERY(float);
+  else if (dtype == kBF16)
+    LS_LATENT_QUERY(bf16_t);
+  else
+    return fail("latent_query: unknown dtype %d", dtype);
+#undef LS_LATENT_QUERY
+  return check_launch("latent_query");
+}
+
+extern "C" int ls_heads_product(int dtype, const void* x, long ldx, int x_stride, const void* w, int H, int N, int K,
+                                int n_rows, void* out, long ldo, int o_stride, void* stream) {
+  LS_REQUIRE(n_rows > 0 && H > 0 && N > 0 && K > 0 && x && w && out, "heads_product: bad sizes");
+  LS_REQUIRE(x_stride >= 0 && o_stride >= 0 && ldx >= (long)(H - 1) * x_stride + K && ldo >= (long)(H - 1) * o_stride + N,
+             "heads_product: the heads do not fit the rows");
+  LS_REQUIRE(dtype == kF32 || dtype == kBF16, "heads_product: unknown dtype %d", dtype);
+  const int vec = dtype == kF32 ? 4 : 8;
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(w) % 16 == 0, "heads_product: the weights must be 16-byte aligned");
+  const int x_aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && ldx % vec == 0 && x_stride % vec == 0 && K % vec == 0;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool many = n_rows > 64;
+  const int rows_a_block = many ? 64 : 16;
+  const dim3 grid((n_rows + rows_a_block - 1) / rows_a_block, H, (N + 63) / 64);
+#define LS_HEADS(T_, RT_)                                                                                            \
+  hipLaunchKernelGGL((heads_product_kernel<T_, RT_>), grid, dim3(256), 0, s, (const T_*)x, ldx, x_stride, (const T_*)w, N, \
+                     K, n_rows, (T_*)out, ldo, o_stride, x_aligned)
+  if (dtype == kF32) {
+    if (many) LS_HEADS(float, 4); else LS_HEADS(float, 1);
+  } else {
+    if (many) LS_HEADS(bf16_t, 4); else LS_HEADS(bf16_t, 1);
+  }
+#undef LS_HEADS
+  return check_launch("heads_product");
+}
+
+extern "C" int ls_delta_max_dim() { return 256; }
+
+// The rows of a head's queries and keys in the scratch buffer: the head size rounded up to what the lanes of the
+// recurrence hold (16, 32, 64, 128 or 256).
+extern "C" int ls_delta_padded_dim(int D) {
+  int dp = 16;
+  while (dp < D) dp *= 2;
+  return dp;
+}
+
+// Floats of scratch that ls_delta_rule needs: qk, vv and gates.
+extern "C" long ls_delta_scratch_floats(int n_tokens, int G, int H, int D, int DV) {
+  return (long)n_tokens * (2L * G * ls_delta_padded_dim(D) + (long)H * DV + 2L * H);
+}
+
+extern "C" int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int H, int D, int DV, int M,
+                             const float* taps, const float* a_log, const float* dt_bias, float unit_eps,
+                             const int* tok_seq, const int* tok_pos, const void* seqs, int n_seqs, float* state,
+                             long state_stride, float* scratch, float* out, long ldo, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && n_seqs > 0 && G > 0 && H > 0 && H % G == 0 && D > 0 && D <= 256 && DV > 0 && M >= 1,
+             "delta_rule: bad sizes (%d key heads, %d heads, keys of %d, values of %d, %d taps)", G, H, D, DV, M);
+  const long C = 2L * G * D + (long)H * DV;
+  const long conv_at = (long)H * D * DV;
+  LS_REQUIRE(ld >= C + 2L * H && state_stride >= conv_at + (long)(M - 1) * C && ldo >= (long)H * DV,
+             "delta_rule: rows or state are too short");
+  LS_REQUIRE(raw && taps && a_log && dt_bias && tok_seq && tok_pos && seqs && state && scratch && out,
+             "delta_rule: null operand");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(scratch) % 16 == 0, "delta_rule: the scratch must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int dp = ls_delta_padded_dim(D);
+  float* qk = scratch;
+  float* vv = qk + (long)n_tokens * 2 * G * dp;
+  float* gates = vv + (long)n_tokens * H * DV;
+  const long units = (long)n_tokens * (2 * G + H + 1);
+  hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, raw, ld, n_tokens, G, H, D, DV,
+                     dp, M, taps, a_log, dt_bias, unit_eps, tok_seq, tok_pos, (const SeqMeta*)seqs, state, state_stride,
+                     conv_at, qk, vv, gates);
+  const dim3 grid(n_seqs * H, (DV + 15) / 16);
+#define LS_DELTA(R_)                                                                                                  \
+  hipLaunchKernelGGL(delta_rule_kernel<R_>, grid, dim3(64), 0, s, qk, vv, gates, G, H, D, DV, (const SeqMeta*)seqs, state, \
+                     state_stride, out, ldo)
+  switch (dp) {
+    case 16: LS_DELTA(4); break;
+    case 32: LS_DELTA(8); break;
+    case 64: LS_DELTA(16); break;
+    case 128: LS_DELTA(32); break;
+    default: LS_DELTA(64); break;
+  }
+#undef LS_DELTA
+  if (M > 1)
+    hipLaunchKernelGGL(delta_conv_state_kernel, dim3(n_seqs, (unsigned)((C + 255) / 256)), dim3(256), 0, s, raw, ld, (int)C,
+                       M, (const SeqMeta*)seqs, state, state_stride, conv_at);
+  return check_launch("delta_rule");
+}

@@ -161,6 +161,7 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 //   v = k as projected, with its bias, before any norm (keys_are_values; DV == D);
 //   q and k each divided by the root mean square over ALL their heads at once (the whole projection is one
 //   vector: x / sqrt(mean(x^2) + eps)), times a weight an element (q_norm [H*D], k_norm [G*D]; null: no norm);
+//   or, with per_head, every head of q and of k divided by its own root mean square over D (no weights);
 //   q and k rotated on their first `rot` dimensions at the token's position, pairs (i, i + rot/2) or, with
 //   `neighbours`, (2i, 2i + 1), angle tables [positions][rot/2];
 //   q -> q_out [T][H*Dp] (T);  k -> key pages [page][G][slot][Dp], Dp >= D with zeros beyond D (a kernel that loads
@@ -169,6 +170,8 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 // is asked for).  The sums of squares: thread t adds the squares of elements t, t + 256, ... in
 // ascending order, then a butterfly over the wave and the wave sums in wave order: a function of the sizes only.
 // ---------------------------------------------------------------------------
+constexpr int kMaxNormedHeads = 1024;  // query and key heads of a projection whose heads are normalised one by one
+
 __device__ __forceinline__ float block_sum256(float v, float* scratch) {
   v = wave_sum(v);
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -180,18 +183,32 @@ __device__ __forceinline__ float block_sum256(float v, float* scratch) {
 
 template <typename T>
 __global__ __launch_bounds__(256) void qkv_post_kernel(
-    const float* __restrict__ raw, long ld, int H, int G, int D, int Dp, int DV, int keys_are_values,
+    const float* __restrict__ raw, long ld, int H, int G, int D, int Dp, int DV, int keys_are_values, int per_head,
     const float* __restrict__ bias, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot, int neighbours,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
     const int* __restrict__ table, int table_stride, T* __restrict__ q_out, long ldq, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int page_size) {
   __shared__ float scratch[4];
+  __shared__ float head_scale[kMaxNormedHeads];
   const int t = blockIdx.x;
   const float* row = raw + (long)t * ld;
   const int pos = tok_pos[t];
   const int nq = H * D, nk = G * D, nv = G * DV;
   float rq = 1.0f, rk = 1.0f;
+  if (per_head) {
+    // a wave a head of q | k: lane i adds the squares of the elements i, i + 64, ... ascending, then a butterfly
+    for (int head = threadIdx.x >> 6; head < H + G; head += 4) {
+      float part = 0.f;
+      for (int i = threadIdx.x & 63; i < D; i += 64) {
+        const float x = row[head * D + i] + (bias ? bias[head * D + i] : 0.f);
+        part = part + x * x;
+      }
+      const float total = wave_sum(part);
+      if ((threadIdx.x & 63) == 0) head_scale[head] = 1.0f / sqrtf(total / (float)D + eps);
+    }
+    __syncthreads();
+  }
   if (q_norm) {
     float part = 0.f;
     for (int e = threadIdx.x; e < nq; e += 256) {
@@ -222,11 +239,13 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     const float r = is_q ? rq : rk;
     float own = row[e] + (bias ? bias[e] : 0.f);
     if (w) own = own * r * w[at];
+    if (per_head) own = own * head_scale[e / D];
     const int i = e % D;
     if (i < rot) {
       const int pe = neighbours ? (e ^ 1) : (i < half ? e + half : e - half);
       float other = row[pe] + (bias ? bias[pe] : 0.f);
       if (w) other = other * r * w[is_q ? pe : pe - nq];
+      if (per_head) other = other * head_scale[e / D];
       const int pair = neighbours ? (i >> 1) : (i < half ? i : i - half);
       const bool lower = neighbours ? (i & 1) == 0 : i < half;
       own = lower ? own * cos_row[pair] - other * sin_row[pair] : own * cos_row[pair] + other * sin_row[pair];
@@ -586,7 +605,7 @@ extern "C" int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, i
 }
 
 extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int Dp, int DV,
-                           int keys_are_values, const float* bias, const float* q_norm, const float* k_norm, float eps,
+                           int keys_are_values, int per_head, const float* bias, const float* q_norm, const float* k_norm, float eps,
                            const float* cos_table, const float* sin_table, int rot, int neighbours,
                            int table_positions, int max_pos, const int* tok_seq, const int* tok_pos, const void* seqs,
                            const int* table, int table_stride, void* q_out, long ldq, void* k_pages, void* v_pages,
@@ -602,13 +621,15 @@ extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, i
              "qkv_post: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
   LS_REQUIRE(max_pos / page_size < table_stride, "qkv_post: position %d is beyond the block table", max_pos);
   LS_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) && (!q_norm || eps > 0.f), "qkv_post: bad norm");
+  LS_REQUIRE(!per_head || (!q_norm && eps > 0.f && H + G <= kMaxNormedHeads),
+             "qkv_post: a norm a head has no weights and takes up to %d heads", kMaxNormedHeads);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   // Without a norm every element stands alone: a thread an element.  With one, every workgroup of a token forms the
   // row's sums itself, so a step of many tokens gives each token one workgroup, and a few tokens are spread out.
   const unsigned all = (unsigned)(((long)(H + G) * Dp + (long)G * DV + 255) / 256);
-  const unsigned pieces = !q_norm ? all : (n_tokens <= 64 ? all : 1u);
+  const unsigned pieces = !(q_norm || per_head) ? all : (n_tokens <= 64 ? all : 1u);
 #define LS_QKV_POST(T_)                                                                                               \
-  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, pieces), dim3(256), 0, s, raw, ld, H, G, D, Dp, DV, keys_are_values, \
+  hipLaunchKernelGGL(qkv_post_kernel<T_>, dim3(n_tokens, pieces), dim3(256), 0, s, raw, ld, H, G, D, Dp, DV, keys_are_values, per_head, \
                      bias, q_norm, k_norm, eps, cos_table, sin_table, rot, neighbours, tok_seq, tok_pos,              \
                      (const SeqMeta*)seqs, table, table_stride, (T_*)q_out, ldq, (T_*)k_pages, (T_*)v_pages, page_size)
   if (dtype == kF32)

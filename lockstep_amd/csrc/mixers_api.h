@@ -32,10 +32,11 @@ int ls_talk_qkv(int dtype, const float* raw, long ld, int n_tokens, int H, int G
 
 // Post pass of an attention projection raw = q | k | v (| more): biases, a root-mean-square norm over the whole of q
 // and of k (weights q_norm [H*D], k_norm [G*D], or null), rotation in pairs (i, i + rot/2) or of neighbours, keys
-// that are also the values (keys_are_values: no v in raw, the biased unnormalised k is stored as v).  Queries and
+// that are also the values (keys_are_values: no v in raw, the biased unnormalised k is stored as v).  per_head: every
+// head of q and of k is divided by its own root mean square over D instead (no weights).  Queries and
 // keys are written with Dp >= D elements a head, zeros beyond D.
 int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, int H, int G, int D, int Dp, int DV, int keys_are_values,
-                const float* bias, const float* q_norm, const float* k_norm, float eps, const float* cos_table,
+                int per_head, const float* bias, const float* q_norm, const float* k_norm, float eps, const float* cos_table,
                 const float* sin_table, int rot, int neighbours, int table_positions, int max_pos, const int* tok_seq,
                 const int* tok_pos, const void* seqs, const int* table, int table_stride, void* q_out, long ldq,
                 void* k_pages, void* v_pages, int page_size, void* stream);
@@ -54,6 +55,45 @@ int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at
 // Per (token, head): x [DV] / sqrt(mean(x^2) + eps), times weight [DV] and silu(gate) where given.
 int ls_head_norm_gate(int out_dtype, const float* x, long ldx, int n_tokens, int H, int DV, const float* weight,
                       const float* gate, long ldg, float eps, void* out, long ldo, void* stream);
+
+// A residual stream of n copies X [rows][n][width] float.  Write (P given): y = P[0][row] + P[1][row] + ..., then
+// X'_t = sum_s mix[s][t] X_s + gain[t] y for all copies at once.  Read (out given): u = sum_t take[t] X'_t (take null:
+// the plain sum), out [n_rows][ld_out] = u / sqrt(mean(u^2) + eps) * weight.  rows: the rows to take, or null.
+int ls_streams_max();
+int ls_streams_max_width();
+int ls_streams_step(int dtype, float* X, long ldx, int n, int width, const float* P, int slices, int p_rows,
+                    const float* mix, const float* gain, const float* take, const float* weight, float eps, void* out,
+                    long ld_out, const int* rows, int n_rows, void* stream);
+
+// Post pass of the down projections of attention over a latent, raw = a (QR) | c (CR) | r (RD): a and c normalised
+// with their weights, r rotated in neighbouring pairs; a -> a_out, c | r -> key pages (heads of Dp elements, one
+// key/value head), c -> value pages.  has_kv 0: a alone.
+int ls_latent_post(int dtype, const float* raw, long ld, int n_tokens, int QR, int CR, int RD, int Dp, int has_kv,
+                   const float* a_weight, const float* c_weight, float eps, const float* cos_table, const float* sin_table,
+                   int rot, int table_positions, int max_pos, const int* tok_seq, const int* tok_pos, const void* seqs,
+                   const int* table, int table_stride, void* a_out, long lda, void* k_pages, void* v_pages, int page_size,
+                   void* stream);
+
+// Post pass of the queries' up projection qf (heads of D plain and RD rotated dimensions): the plain part to
+// plain_out [T][H*D], the rotated part, rotated, to q_out [T][H*Dp] behind the CR dimensions of the latent.
+int ls_latent_query(int dtype, const float* qf, long ld, int n_tokens, int H, int D, int RD, int CR, int Dp,
+                    const float* cos_table, const float* sin_table, int rot, int table_positions, int max_pos,
+                    const int* tok_pos, void* plain_out, long ldp, void* q_out, long ldq, void* stream);
+
+// out[t][head * o_stride + n] = sum_k w[head][n][k] x[t][head * x_stride + k]; w [H][N][K], x and out of one dtype.
+int ls_heads_product(int dtype, const void* x, long ldx, int x_stride, const void* w, int H, int N, int K, int n_rows,
+                     void* out, long ldo, int o_stride, void* stream);
+
+// The gated delta rule over the tokens of every request of the step (see latent_delta.hip).  raw float = q (G heads of
+// D) | k (G of D) | v (H of DV) | b (H) | a (H) | ...; state [slots][state_stride] float = S [H][D][DV], then the
+// last M - 1 inputs of the convolutions [M - 1][2 G D + H DV]; taps [2 G D + H DV][M]; out [T][ldo] float gets o_t.
+int ls_delta_max_dim();
+int ls_delta_padded_dim(int D);
+long ls_delta_scratch_floats(int n_tokens, int G, int H, int D, int DV);
+int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int H, int D, int DV, int M, const float* taps,
+                  const float* a_log, const float* dt_bias, float unit_eps, const int* tok_seq, const int* tok_pos,
+                  const void* seqs, int n_seqs, float* state, long state_stride, float* scratch, float* out, long ldo,
+                  void* stream);
 
 int ls_listed_index(const char* name);
 int ls_call_listed(int index, const long long* words, int n);

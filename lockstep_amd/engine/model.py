@@ -192,7 +192,7 @@ class Model:
 
     def _forward(self, ctx: StepContext, logits=None):
         """Launch the step's kernels on the current stream."""
-        h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size), torch.float32)
+        h = ctx.buf("residual", (ctx.n_tokens, self.spec.hidden_size * self.spec.residual_copies), torch.float32)
         self.embedding.forward(ctx, ctx.token_ids, h)
         pending = None          # an addition to h that a layer left to the next reader of h
         kernels = self.rt.kernels

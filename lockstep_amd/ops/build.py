@@ -48,7 +48,7 @@ FLAGS = [
 ]
 CORE_SOURCES = ("core.hip", "gemm.hip", "sample.hip")
 ATTENTION_SOURCES = ("attention.hip",)
-MIXERS_SOURCES = ("mixers.hip",)
+MIXERS_SOURCES = ("mixers.hip", "latent_delta.hip")
 TALKING_SOURCES = ("talking_attention.hip",)
 SINK_SOURCES = ("sink_attention.hip",)
 EXPERTS_SOURCES = ("experts.hip",)

@@ -954,13 +954,14 @@ class Kernels:
     def qkv_post(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, q_norm,
                  k_norm, eps: float, cos, sin, rot: int, neighbours: bool, max_pos: int, tok_seq, tok_pos, seqs, table,
                  q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False,
-                 key_pad: int | None = None) -> None:
+                 key_pad: int | None = None, per_head: bool = False) -> None:
         """Post pass of the fused projection ``raw`` (float32, ``q | k | v | ...``; no ``v`` with
         ``keys_are_values``, where the biased, unnormalised keys are stored as the values): biases, a
         root-mean-square norm over the whole of q and of k with the weights ``q_norm`` / ``k_norm``, rotation of
         the first ``rot`` dimensions of each head in pairs ``(i, i + rot/2)`` or of ``neighbours``, queries to
         ``q_out``, keys and values to their pages.  ``key_pad``: the size of a head in ``q_out`` and in the key
-        pages where it exceeds ``dim`` (zeros beyond ``dim``)."""
+        pages where it exceeds ``dim`` (zeros beyond ``dim``).  ``per_head``: every head of q and of k is divided
+        by its own root mean square over ``dim`` (``eps`` inside the root, no weights) instead."""
         _rows_ok(raw, "qkv_post raw"); _rows_ok(q_out, "qkv_post q_out")
         key_pad = dim if key_pad is None else key_pad
         width = heads * dim + kv_heads * dim + (0 if keys_are_values else kv_heads * vdim)
@@ -976,6 +977,8 @@ class Kernels:
             raise KernelError("qkv_post normalises both q and k or neither")
         if q_norm is not None:
             self._f32_vector(q_norm, heads * dim, "qkv_post q_norm"); self._f32_vector(k_norm, kv_heads * dim, "qkv_post k_norm")
+        if per_head and (q_norm is not None or not eps > 0):
+            raise KernelError("qkv_post: a norm a head takes no weights and needs a positive eps")
         positions = self._rotation_tables(cos, sin, rot, max_pos)
         self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, key_pad, vdim)
         if not (max_pos // page_size < table.shape[1]):
@@ -988,7 +991,7 @@ class Kernels:
         lib = self.mixers_lib()
         self._launch(lib, lib.ls_qkv_post, (
             c_int(DTYPE_CODE[q_out.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(heads),
-            c_int(kv_heads), c_int(dim), c_int(key_pad), c_int(vdim), c_int(int(keys_are_values)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
+            c_int(kv_heads), c_int(dim), c_int(key_pad), c_int(vdim), c_int(int(keys_are_values)), c_int(int(per_head)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
             c_float(eps), _ptr(cos), _ptr(sin), c_int(rot), c_int(int(neighbours)), c_int(positions), c_int(max_pos),
             _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1]), _ptr(q_out),
             c_long(q_out.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size), _stream()))
@@ -1102,9 +1105,11 @@ class Kernels:
 
     def experts_apply(self, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top: int,
                       rows_a_tile: int, order: torch.Tensor, tiles: torch.Tensor, weight: torch.Tensor, limit: float,
-                      alpha: float, act: torch.Tensor, partials: torch.Tensor) -> None:
+                      alpha: float, act: torch.Tensor, partials: torch.Tensor, shift: float = 1.0) -> None:
         """``partials[k][t] = weight[t, k] * down_e(act(gate_e x[t], up_e x[t]))`` for every token's ``k``-th
-        expert ``e``, with the clamped gated unit of ``glu_clamped`` as activation.  ``w_gate``, ``w_up``
+        expert ``e``, with the clamped gated unit of ``glu_clamped`` as activation (``min(g, limit) sigmoid(alpha
+        min(g, limit)) (clamp(u, -limit, limit) + shift)``; an infinite ``limit``, ``alpha`` 1 and ``shift`` 0 are the
+        plain unit ``silu(g) u``).  ``w_gate``, ``w_up``
         ``[E, F, K]``, ``w_down [E, N, F]`` in the compute dtype; ``act``: scratch ``[T * top, F]`` of the
         compute dtype; ``partials [top, T, N]`` float32; the routing as ``experts_route`` left it."""
         _rows_ok(x, "experts_apply x"); _rows_ok(act, "experts_apply act")
@@ -1130,7 +1135,215 @@ class Kernels:
         self._launch(lib, lib.ls_experts_apply, (
             c_int(DTYPE_CODE[x.dtype]), _ptr(x), c_long(x.stride(0)), _ptr(w_gate), _ptr(w_up), _ptr(w_down), c_int(t),
             c_int(e), c_int(top), c_int(k), c_int(f), c_int(n), c_int(rows_a_tile), _ptr(order), _ptr(tiles), c_int(cap),
-            _ptr(weight), c_float(limit), c_float(alpha), _ptr(act), c_long(act.stride(0)), _ptr(partials), _stream()))
+            _ptr(weight), c_float(limit), c_float(alpha), c_float(shift), _ptr(act), c_long(act.stride(0)), _ptr(partials),
+            _stream()))
+
+    def experts_route_table(self, token_ids: torch.Tensor, table: torch.Tensor, experts: int, rows_a_tile: int,
+                            expert: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, tiles: torch.Tensor,
+                            counts: torch.Tensor) -> None:
+        """Routing without a router: token ``t`` uses the experts in row ``token_ids[t]`` of ``table [vocab, top]``
+        (int32, entries in ``[0, experts)``, those of a row differ), each with the weight ``1 / top``.  The
+        outputs are those of ``experts_route``."""
+        if not (table.is_cuda and table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()):
+            raise KernelError("experts_route_table table must be int32 [vocab, top] on the GPU")
+        t, top = token_ids.shape[0], table.shape[1]
+        if not (0 < top <= experts):
+            raise KernelError(f"experts_route_table: {top} experts a token of {experts}")
+        self._i32(token_ids, t, "experts_route_table token_ids")
+        cap = self.experts_tile_capacity(t, experts, top, rows_a_tile)
+        self._i32(expert, t * top, "experts_route_table expert"); self._i32(order, t * top, "experts_route_table order")
+        self._i32(tiles, 4 * cap, "experts_route_table tiles"); self._i32(counts, experts, "experts_route_table counts")
+        if not (weight.is_cuda and weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() >= t * top):
+            raise KernelError("experts_route_table weight must be float32 [T, top]")
+        if t == 0:
+            return
+        lib = self.experts_lib()
+        self._launch(lib, lib.ls_experts_route_table, (
+            _ptr(token_ids), _ptr(table), c_int(t), c_int(experts), c_int(top), c_int(rows_a_tile), _ptr(expert),
+            _ptr(weight), _ptr(order), _ptr(tiles), c_int(cap), _ptr(counts), _stream()))
+
+    # -- a residual stream of several copies ------------------------------------------------------
+    def streams_max(self) -> tuple[int, int]:
+        """(the most copies, the widest row) that ``streams_step`` takes."""
+        return self._memo(("streams_max",), lambda: (int(self.mixers_lib().ls_streams_max()),
+                                                     int(self.mixers_lib().ls_streams_max_width())))
+
+    def streams_step(self, x: torch.Tensor, copies: int, partials, mix, gain, take, weight, eps: float, out,
+                     rows: torch.Tensor | None = None) -> None:
+        """One step of a residual stream of ``copies`` copies, ``x`` float32 ``[T, copies * width]``.  With
+        ``partials [slices, T, width]`` (a sublayer's output as slice sums) the copies are rewritten:
+        ``x'_t = sum_s mix[s, t] x_s + gain[t] y``, ``y`` the sum of the slices in ascending order.  With ``out
+        [rows, width]`` the copies are then read: ``u = sum_t take[t] x'_t`` (``take`` None: their plain sum) and
+        ``out = u / sqrt(mean(u^2) + eps) * weight``.  ``rows`` selects rows of ``x`` (all without it)."""
+        _rows_ok(x, "streams_step x")
+        if not (x.dtype == torch.float32 and copies > 0 and x.shape[1] % copies == 0):
+            raise KernelError("streams_step works on float32 rows of whole copies")
+        width = x.shape[1] // copies
+        most, widest = self.streams_max()
+        if not (copies <= most and width <= widest):
+            raise KernelError(f"streams_step takes up to {most} copies of up to {widest} elements, got {copies} of {width}")
+        n_rows = x.shape[0] if rows is None else rows.shape[0]
+        if rows is not None and not (rows.is_cuda and rows.dtype == torch.int32 and rows.is_contiguous()):
+            raise KernelError("streams_step rows: int32 on the GPU")
+        slices = p_rows = 0
+        if partials is not None:
+            if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and partials.dim() == 3
+                    and partials.shape[2] == width and partials.shape[1] >= x.shape[0]):
+                raise KernelError(f"streams_step partials must be float32 [slices, >= {x.shape[0]}, {width}]")
+            slices, p_rows = partials.shape[0], partials.shape[1]
+            self._f32_vector(mix, copies * copies, "streams_step mix"); self._f32_vector(gain, copies, "streams_step gain")
+        if take is not None:
+            self._f32_vector(take, copies, "streams_step take")
+        dtype, ld_out = torch.float32, 0
+        if out is not None:
+            _rows_ok(out, "streams_step out")
+            if not (out.dtype in DTYPE_CODE and tuple(out.shape) == (n_rows, width) and eps > 0):
+                raise KernelError(f"streams_step out must be [{n_rows},{width}], eps positive")
+            self._f32_vector(weight, width, "streams_step weight")
+            dtype, ld_out = out.dtype, out.stride(0)
+        elif partials is None:
+            return
+        if n_rows == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_streams_step, (
+            c_int(DTYPE_CODE[dtype]), _ptr(x), c_long(x.stride(0)), c_int(copies), c_int(width), _ptr(partials),
+            c_int(slices), c_int(p_rows), _ptr(mix), _ptr(gain), _ptr(take), _ptr(weight), c_float(eps), _ptr(out),
+            c_long(ld_out), _ptr(rows), c_int(n_rows), _stream()))
+
+    # -- attention over a cached latent: the passes around it ----------------------------------------
+    def latent_post(self, raw: torch.Tensor, n_tokens: int, q_rank: int, kv_rank: int, rot_dim: int, key_pad: int,
+                    has_kv: bool, q_weight, kv_weight, eps: float, cos, sin, rot: int, max_pos: int, tok_seq, tok_pos,
+                    seqs, table, q_latent: torch.Tensor, k_pages, v_pages, page_size: int) -> None:
+        """Post pass of the down projections ``raw`` (float32, ``a | c | r``): the query latent ``a`` normalised
+        with ``q_weight`` into ``q_latent``; with ``has_kv`` the latent ``c`` normalised with ``kv_weight`` into the
+        key pages (dimensions ``0 .. kv_rank`` of the one key head of ``key_pad`` elements) and into the value
+        pages, and the shared key part ``r``, rotated in neighbouring pairs on its first ``rot`` dimensions,
+        behind it in the key pages."""
+        _rows_ok(raw, "latent_post raw"); _rows_ok(q_latent, "latent_post q_latent")
+        width = q_rank + (kv_rank + rot_dim if has_kv else 0)
+        if not (raw.dtype == torch.float32 and raw.shape[0] >= n_tokens and raw.shape[1] >= width):
+            raise KernelError(f"latent_post raw must be float32 [>= {n_tokens}, >= {width}]")
+        if not (q_latent.dtype in DTYPE_CODE and q_latent.shape[0] >= n_tokens and q_latent.shape[1] == q_rank):
+            raise KernelError("latent_post q_latent has the wrong shape or dtype")
+        self._f32_vector(q_weight, q_rank, "latent_post q_weight")
+        positions = 0
+        if has_kv:
+            self._f32_vector(kv_weight, kv_rank, "latent_post kv_weight")
+            positions = self._rotation_tables(cos, sin, rot, max_pos)
+            self._paged_ok(k_pages, v_pages, table, q_latent.dtype, 1, page_size, key_pad, kv_rank)
+            if not (key_pad >= kv_rank + rot_dim and max_pos // page_size < table.shape[1]):
+                raise KernelError("latent_post: the key head is too short, or a position lies beyond the block table")
+            for name, t in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+                if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n_tokens):
+                    raise KernelError(f"{name} must be int32 with at least {n_tokens} entries")
+        if n_tokens == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_latent_post, (
+            c_int(DTYPE_CODE[q_latent.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(q_rank),
+            c_int(kv_rank), c_int(rot_dim), c_int(key_pad), c_int(int(has_kv)), _ptr(q_weight),
+            _ptr(kv_weight if has_kv else None), c_float(eps), _ptr(cos if has_kv else None), _ptr(sin if has_kv else None),
+            c_int(rot), c_int(positions), c_int(max_pos), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs),
+            _ptr(table if has_kv else None), c_int(table.shape[1] if has_kv else 0), _ptr(q_latent),
+            c_long(q_latent.stride(0)), _ptr(k_pages if has_kv else None), _ptr(v_pages if has_kv else None),
+            c_int(page_size), _stream()))
+
+    def latent_query(self, qf: torch.Tensor, n_tokens: int, heads: int, dim: int, rot_dim: int, kv_rank: int, key_pad: int,
+                     cos, sin, rot: int, max_pos: int, tok_pos, plain: torch.Tensor, q_out: torch.Tensor) -> None:
+        """Post pass of the queries' up projection ``qf`` (float32, heads of ``dim`` plain and ``rot_dim`` rotated
+        dimensions): the plain parts into ``plain [T, heads*dim]``; the rotated parts, rotated in neighbouring
+        pairs on their first ``rot`` dimensions, into ``q_out [T, heads*key_pad]`` behind the ``kv_rank``
+        dimensions of each head that the product with the keys' up projection fills (zeros up to ``key_pad``)."""
+        _rows_ok(qf, "latent_query qf"); _rows_ok(plain, "latent_query plain"); _rows_ok(q_out, "latent_query q_out")
+        if not (qf.dtype == torch.float32 and qf.shape[0] >= n_tokens and qf.shape[1] == heads * (dim + rot_dim)):
+            raise KernelError(f"latent_query qf must be float32 [>= {n_tokens}, {heads * (dim + rot_dim)}]")
+        if not (plain.dtype in DTYPE_CODE and q_out.dtype == plain.dtype and plain.shape[0] >= n_tokens
+                and plain.shape[1] == heads * dim and q_out.shape[0] >= n_tokens and q_out.shape[1] == heads * key_pad
+                and key_pad >= kv_rank + rot_dim):
+            raise KernelError("latent_query outputs have the wrong shape or dtype")
+        positions = self._rotation_tables(cos, sin, rot, max_pos)
+        if not (tok_pos.is_cuda and tok_pos.dtype == torch.int32 and tok_pos.is_contiguous() and tok_pos.numel() >= n_tokens):
+            raise KernelError("latent_query tok_pos: int32, one position a token")
+        if n_tokens == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_latent_query, (
+            c_int(DTYPE_CODE[plain.dtype]), _ptr(qf), c_long(qf.stride(0)), c_int(n_tokens), c_int(heads), c_int(dim),
+            c_int(rot_dim), c_int(kv_rank), c_int(key_pad), _ptr(cos), _ptr(sin), c_int(rot), c_int(positions),
+            c_int(max_pos), _ptr(tok_pos), _ptr(plain), c_long(plain.stride(0)), _ptr(q_out), c_long(q_out.stride(0)),
+            _stream()))
+
+    def heads_product(self, x: torch.Tensor, x_stride: int, w: torch.Tensor, out: torch.Tensor, o_stride: int,
+                      n_rows: int | None = None) -> None:
+        """A product a head: ``out[t, h * o_stride + n] = sum_k w[h, n, k] x[t, h * x_stride + k]`` with
+        ``w [heads, N, K]`` contiguous; ``x``, ``w`` and ``out`` in one compute dtype."""
+        _rows_ok(x, "heads_product x"); _rows_ok(out, "heads_product out")
+        n_rows = x.shape[0] if n_rows is None else n_rows
+        if not (w.is_cuda and w.dim() == 3 and w.is_contiguous() and w.dtype in DTYPE_CODE and x.dtype == w.dtype == out.dtype):
+            raise KernelError("heads_product w must be [heads, N, K] contiguous, all operands of one dtype")
+        heads, n, k = w.shape
+        if not (x.shape[0] >= n_rows and out.shape[0] >= n_rows and x.shape[1] >= (heads - 1) * x_stride + k
+                and out.shape[1] >= (heads - 1) * o_stride + n and x_stride >= 0 and o_stride >= 0):
+            raise KernelError("heads_product: the heads do not fit the rows")
+        if n_rows == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_heads_product, (
+            c_int(DTYPE_CODE[w.dtype]), _ptr(x), c_long(x.stride(0)), c_int(x_stride), _ptr(w), c_int(heads), c_int(n),
+            c_int(k), c_int(n_rows), _ptr(out), c_long(out.stride(0)), c_int(o_stride), _stream()))
+
+    # -- the gated delta rule -----------------------------------------------------------------------
+    def delta_max_dim(self) -> int:
+        return self._memo(("delta_max_dim",), lambda: int(self.mixers_lib().ls_delta_max_dim()))
+
+    def delta_scratch_floats(self, n_tokens: int, kv_heads: int, heads: int, dim: int, vdim: int) -> int:
+        lib = self.mixers_lib()
+        lib.ls_delta_scratch_floats.restype = ctypes.c_long
+        return int(lib.ls_delta_scratch_floats(c_int(n_tokens), c_int(kv_heads), c_int(heads), c_int(dim), c_int(vdim)))
+
+    def delta_rule(self, raw: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int, taps: torch.Tensor, a_log,
+                   dt_bias, unit_eps: float, tok_seq, tok_pos, seqs, n_seqs: int, state: torch.Tensor,
+                   scratch: torch.Tensor, out: torch.Tensor) -> None:
+        """The gated delta rule over the tokens of every request of the step.  ``raw`` float32 holds the
+        projections ``q | k`` (``kv_heads`` heads of ``dim``) ``| v`` (``heads`` of ``vdim``) ``| b | a``
+        (``heads`` each); every channel of q, k and v passes a causal convolution with ``taps [channels, M]``
+        (the last column is the current token's) and silu; q and k become unit vectors (``unit_eps`` inside
+        the root), q also times ``dim^-1/2``; ``beta = sigmoid(b)``, ``decay = exp(-exp(a_log) softplus(a +
+        dt_bias))``; per head ``S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``.  ``state``
+        float32 ``[slots, heads*dim*vdim + (M-1)*channels]``: the matrices, then the convolutions' last inputs;
+        read and left for the next step.  ``out`` float32 ``[T, heads*vdim]``."""
+        _rows_ok(raw, "delta_rule raw"); _rows_ok(out, "delta_rule out")
+        t = raw.shape[0]
+        channels = 2 * kv_heads * dim + heads * vdim
+        if not (raw.dtype == torch.float32 and raw.shape[1] >= channels + 2 * heads and out.dtype == torch.float32
+                and tuple(out.shape) == (t, heads * vdim)):
+            raise KernelError("delta_rule reads and writes float32 rows, out [T, heads*vdim]")
+        if not (heads % kv_heads == 0 and dim <= self.delta_max_dim()):
+            raise KernelError(f"delta_rule: {heads} heads over {kv_heads} key heads, keys of at most {self.delta_max_dim()}")
+        if not (taps.is_cuda and taps.dtype == torch.float32 and taps.is_contiguous() and taps.dim() == 2
+                and taps.shape[0] == channels and taps.shape[1] >= 1):
+            raise KernelError(f"delta_rule taps must be float32 [{channels}, M]")
+        m = taps.shape[1]
+        self._f32_vector(a_log, heads, "delta_rule a_log"); self._f32_vector(dt_bias, heads, "delta_rule dt_bias")
+        if not (state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2
+                and state.shape[1] == heads * dim * vdim + (m - 1) * channels):
+            raise KernelError(f"delta_rule state must be float32 [slots, {heads * dim * vdim + (m - 1) * channels}]")
+        if not (scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous()
+                and scratch.numel() >= self.delta_scratch_floats(t, kv_heads, heads, dim, vdim)):
+            raise KernelError("delta_rule scratch: float32 of delta_scratch_floats elements")
+        for name, v in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous() and v.numel() >= t):
+                raise KernelError(f"delta_rule {name}: int32, one entry a token")
+        if n_seqs == 0 or t == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_delta_rule, (
+            _ptr(raw), c_long(raw.stride(0)), c_int(t), c_int(kv_heads), c_int(heads), c_int(dim), c_int(vdim), c_int(m),
+            _ptr(taps), _ptr(a_log), _ptr(dt_bias), c_float(unit_eps), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs),
+            c_int(n_seqs), _ptr(state), c_long(state.stride(0)), _ptr(scratch), _ptr(out), c_long(out.stride(0)),
+            _stream()))
+
 
 ATTENTION_ITEM_INTS = 32
 COMBINE_ITEM_INTS = 8

@@ -3,7 +3,7 @@
 from .base import (Arrangement, FeedForward, Mixer, Norm, PagedKVSpec, Part, PositionEncoding,
                    StateSpec, WeightSpec, build_part, bump_device_epoch, part_class, register_part,
                    unregister_part)
-from . import attention, block, embedding, experts, mlp, norm, recurrence, rope, sink_attention, talking_attention  # noqa: F401 - register the built-in kinds
+from . import attention, block, embedding, experts, latent_attention, mlp, norm, recurrence, rope, sink_attention, talking_attention  # noqa: F401 - register the built-in kinds
 
 __all__ = ["Arrangement", "FeedForward", "Mixer", "Norm", "PagedKVSpec", "Part", "PositionEncoding",
            "StateSpec", "WeightSpec", "build_part", "bump_device_epoch", "part_class", "register_part",

@@ -49,7 +49,8 @@ class WeightSpec:
     32-bit arithmetic and are kept in float32; ``int`` tensors are integer
     tables kept as int32.  ``init`` steers the random-weights mode: ``normal``
     is N(0, std), ``norm`` is 1 + N(0, norm_std), ``zeros`` is 0, ``identity`` is I + N(0, std) (a
-    square matrix), ``unit`` is uniform in (0, 1).  A dimension of -1 in ``shape`` is one that the
+    square matrix), ``unit`` is uniform in (0, 1), ``around_zero`` is N(0, norm_std) (a norm weight stored
+    as its distance from one), ``distinct`` (an ``int`` table) fills every row with different numbers below ``free``.  A dimension of -1 in ``shape`` is one that the
     checkpoint decides (a table whose number of rows no configuration key gives); random weights
     take ``free`` there.
     """

@@ -120,3 +120,159 @@ class PreNormResidual(Arrangement):
             else:
                 left = self.feed_forward.forward(ctx, x, h, accumulate=True)
         return left if isinstance(left, PendingAdd) else None
+
+
+class PendingWrite(PendingAdd):
+    """A sublayer's output that still has to be written into a residual stream of several copies:
+    ``x'_t = sum_s mix[s, t] x_s + gain[t] y`` with ``y`` the sum of ``partials`` in ascending order.
+    The next reader of the stream does it on its way (the next sublayer's read, or the final norm)."""
+
+    def __init__(self, partials, mix, gain, copies: int):
+        super().__init__(partials)
+        self.mix, self.gain, self.copies = mix, gain, copies
+
+    def flush(self, ctx, stream, rows=None) -> None:
+        ctx.rt.kernels.streams_step(stream, self.copies, self.partials, self.mix, self.gain, None, None, 0.0, None, rows)
+
+
+@register_part("hyper_connections")
+class HyperConnections(Arrangement):
+    """A layer over a residual stream of ``copies`` copies ``x_1 .. x_n`` (``h [T, copies * width]``, all
+    equal to the embedding at the start; the model's last norm reads their sum).  Each sublayer
+    ``f`` (the mixer, then the feed-forward, if any) with its norm reads one weighted sum and writes to
+    all copies at once:
+
+        u = sum_s take[s] x_s;   y = f(norm(u));   x'_t = sum_s mix[s, t] x_s + gain[t] y
+
+    ``mix`` is indexed ``[from, to]``.  The write of a sublayer is left to the launch that reads the
+    stream next, which also normalises what it read: one launch a sublayer.
+
+    Parameters: ``copies``; ``mixer_prefix``, ``feed_forward_prefix``, ``mixer_norm_name``,
+    ``feed_forward_norm_name`` as for ``prenorm_residual``; ``mixer_streams_prefix``,
+    ``feed_forward_streams_prefix``: below them the tensors ``in [n]`` (take), ``out [n]`` (gain) and
+    ``mix [n, n]``.  The norms must be ``rmsnorm`` parts (their weight and eps are applied by the read)."""
+
+    graph_safe = True
+
+    #: steps of at most this many tokens ask their sublayers for slice sums (the write adds them up)
+    SLICE_ROWS = 256
+
+    def __init__(self, layer_spec, prefix: str = ""):
+        super().__init__(layer_spec, build_part)
+        p = layer_spec.arrangement.params
+        base = layer_spec.prefix
+        self.copies = int(p["copies"])
+        if self.copies < 1:
+            raise ValueError(f"a residual stream of {self.copies} copies")
+        self.mixer_norm = build_part(layer_spec.part("mixer_norm"), self.join(base, p["mixer_norm_name"]))
+        self._mixer = build_part(layer_spec.part("mixer"), self.join(base, p["mixer_prefix"]))
+        self.feed_forward = self.feed_forward_norm = None
+        if layer_spec.has("feed_forward"):
+            self.feed_forward_norm = build_part(layer_spec.part("feed_forward_norm"),
+                                                self.join(base, p["feed_forward_norm_name"]))
+            self.feed_forward = build_part(layer_spec.part("feed_forward"), self.join(base, p["feed_forward_prefix"]))
+        for norm in (self.mixer_norm, self.feed_forward_norm):
+            if norm is not None and getattr(norm, "kind", "") != "rmsnorm":
+                raise ValueError("the sublayers of a stream of several copies are normalised by rmsnorm parts")
+        self._defer_mixer = takes(self._mixer.forward, "defer")
+        self._defer_ff = self.feed_forward is not None and takes(self.feed_forward.forward, "defer")
+        self.streams = {}        # sublayer -> (take, gain, mix) on the device
+
+    @classmethod
+    def _stream_specs(cls, prefix: str, n: int, optional: bool = False):
+        from .base import WeightSpec
+
+        return [WeightSpec(f"{prefix}.in", (n,), kind="vector", init="unit", optional=optional),
+                WeightSpec(f"{prefix}.out", (n,), kind="vector", init="norm", optional=optional),
+                WeightSpec(f"{prefix}.mix", (n, n), kind="vector", init="identity", optional=optional)]
+
+    @classmethod
+    def weight_specs(cls, layer_spec, prefix: str = ""):
+        from .base import part_class
+
+        p = layer_spec.arrangement.params
+        base, n = layer_spec.prefix, int(p["copies"])
+        out = []
+        wired = [(layer_spec.part("mixer_norm"), p["mixer_norm_name"]), (layer_spec.part("mixer"), p["mixer_prefix"])]
+        out += cls._stream_specs(cls.join(base, p["mixer_streams_prefix"]), n)
+        if layer_spec.has("feed_forward"):
+            wired += [(layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]),
+                      (layer_spec.part("feed_forward"), p["feed_forward_prefix"])]
+            out += cls._stream_specs(cls.join(base, p["feed_forward_streams_prefix"]), n)
+        else:
+            # what the checkpoint may hold for a second half that never runs is accepted, never used
+            if layer_spec.has("feed_forward_norm"):
+                wired.append((layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]))
+            out += cls._stream_specs(cls.join(base, p["feed_forward_streams_prefix"]), n, optional=True)
+        for spec, name in wired:
+            out += part_class(spec.kind).weight_specs(spec, cls.join(base, name))
+        return out
+
+    def parts(self):
+        if self.feed_forward is None:
+            return (self.mixer_norm, self._mixer)
+        return (self.mixer_norm, self._mixer, self.feed_forward_norm, self.feed_forward)
+
+    @property
+    def mixer(self):
+        return self._mixer
+
+    def load(self, weights, rt) -> None:
+        for part in self.parts():
+            part.load(weights, rt)
+        p = self.layer_spec.arrangement.params
+        most, widest = rt.kernels.streams_max()
+        if self.copies > most:
+            raise ValueError(f"a residual stream of {self.copies} copies; the kernel takes up to {most}")
+        names = [("mixer", p["mixer_streams_prefix"])]
+        if self.feed_forward is not None:
+            names.append(("feed_forward", p["feed_forward_streams_prefix"]))
+        for sublayer, name in names:
+            full = self.join(self.layer_spec.prefix, name)
+            self.streams[sublayer] = tuple(rt.vector(weights.get(f"{full}.{t}").reshape(-1)) for t in ("in", "out", "mix"))
+
+    def _run(self, ctx, sublayer, defers: bool, call, width: int):
+        """One sublayer's output as slice sums ``[slices, T, width]``."""
+        import torch
+
+        t = ctx.n_tokens
+        y = ctx.buf(f"streams.y.{sublayer}", (t, width), torch.float32)
+        if defers and t <= self.SLICE_ROWS:
+            # (a part that does not leave its product as slice sums after all adds it to zeros)
+            y.zero_()
+            left = call(y, True, True)
+            if isinstance(left, PendingAdd):
+                return left.partials
+        else:
+            call(y, False, False)
+        return y.view(1, t, width)
+
+    def forward(self, ctx, run, h, pending=None):
+        """``pending``: the write the previous layer left (a ``PendingWrite``).  Returns this layer's last one."""
+        rt = ctx.rt
+        k = rt.kernels
+        n = self.copies
+        width = h.shape[1] // n
+        if pending is not None and not isinstance(pending, PendingWrite):
+            pending.flush(ctx, h)
+            pending = None
+        take, gain, mix = self.streams["mixer"]
+        x = ctx.buf("block.normed", (ctx.n_tokens, width), rt.dtype)
+        k.streams_step(h, n, None if pending is None else pending.partials, None if pending is None else pending.mix,
+                       None if pending is None else pending.gain, take, self.mixer_norm.weight, self.mixer_norm.eps, x)
+        if self._defer_mixer:
+            call = lambda y, acc, defer: self._mixer.forward(ctx, run, x, y, accumulate=acc, defer=defer)  # noqa: E731
+        else:
+            call = lambda y, acc, defer: self._mixer.forward(ctx, run, x, y, accumulate=acc)  # noqa: E731
+        left = PendingWrite(self._run(ctx, "mixer", self._defer_mixer, call, width), mix, gain, n)
+        if self.feed_forward is None:
+            return left
+        take, gain, mix = self.streams["feed_forward"]
+        x = ctx.buf("block.normed", (ctx.n_tokens, width), rt.dtype)
+        k.streams_step(h, n, left.partials, left.mix, left.gain, take, self.feed_forward_norm.weight,
+                       self.feed_forward_norm.eps, x)
+        if self._defer_ff:
+            call = lambda y, acc, defer: self.feed_forward.forward(ctx, x, y, accumulate=acc, defer=defer)  # noqa: E731
+        else:
+            call = lambda y, acc, defer: self.feed_forward.forward(ctx, x, y, accumulate=acc)  # noqa: E731
+        return PendingWrite(self._run(ctx, "feed_forward", self._defer_ff, call, width), mix, gain, n)

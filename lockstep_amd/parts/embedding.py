@@ -11,7 +11,8 @@ from .base import Part, WeightSpec, register_part
 class TokenEmbedding(Part):
     """``h[t] = E[token[t]] * scale``; without ``scale`` no scaling (reference
     engine/model/qwen3.py:319).  Parameters: ``name``, ``vocab_size``, ``hidden_size``,
-    ``scale`` (optional)."""
+    ``scale`` (optional), ``copies`` (optional: the residual stream holds that many copies of a row,
+    ``[T, copies * hidden_size]``, which all start as the embedding)."""
 
     graph_safe = True
 
@@ -19,6 +20,7 @@ class TokenEmbedding(Part):
         super().__init__(spec, prefix)
         self.table = None
         self.scale = float(spec.params.get("scale", 1.0))
+        self.copies = int(spec.params.get("copies") or 1)
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
@@ -28,7 +30,9 @@ class TokenEmbedding(Part):
         self.table = rt.matrix(weights.get(self.spec["name"]), share_key=weights.source_name(self.spec["name"]))
 
     def forward(self, ctx, tokens, out) -> None:
-        ctx.rt.kernels.embed(tokens, self.table, out, self.scale)
+        width = self.table.shape[1]
+        for c in range(self.copies):
+            ctx.rt.kernels.embed(tokens, self.table, out[:, c * width:(c + 1) * width] if self.copies > 1 else out, self.scale)
 
 
 @register_part("linear_head")

@@ -6,8 +6,12 @@ that every token uses.
     w[t, k]   = softmax over the chosen logits alone
     out[t]    = sum_k w[t, k] * expert_chosen(t)[k](x[t])  +  shared(x[t])
 
+With ``router = "table"`` there is no router: row ``token id`` of an integer table ``[vocab, top]`` names
+the token's experts (the entries of a row differ) and each weighs ``1 / top``.
+
 Every expert is the clamped gated unit of ``clamped_gated_mlp`` (``down(g sigmoid(alpha g) (u + 1))``,
-``g = min(gate x, limit)``, ``u = clamp(up x, -limit, limit)``) without biases; the shared expert is a
+``g = min(gate x, limit)``, ``u = clamp(up x, -limit, limit)``) without biases, or, without a ``limit``,
+the plain gated unit ``down(silu(gate x) * (up x))``; the shared expert is a
 ``clamped_gated_mlp`` part with sizes and constants of its own.  Routing, grouping of the tokens by
 expert and the experts' products all run on the device (csrc/experts.hip), so a decode step can be
 replayed from a graph.  The result is left as ``top`` (+ 1) slices, one for a token's k-th expert
@@ -31,7 +35,9 @@ class RoutedExperts(FeedForward):
     """Parameters: ``hidden_size``, ``intermediate_size`` (of one expert), ``experts``, ``top``, ``limit``,
     ``alpha``, ``shared`` (None or the ``PartSpec`` of a feed-forward that runs for every token, built
     below ``<prefix>.shared``).  Tensors below the prefix: ``e<i>.gate``, ``e<i>.up`` ``[F, H]``,
-    ``e<i>.down`` ``[H, F]`` for every expert ``i``, ``router`` ``[E, H]`` and ``router.b`` ``[E]``."""
+    ``e<i>.down`` ``[H, F]`` for every expert ``i``, ``router`` ``[E, H]`` and ``router.b`` ``[E]``.
+    ``limit`` None: the plain gated unit with SiLU.  ``router`` ``"table"`` (default ``"linear"``): the
+    tensor ``table`` ``[vocab_size, top]`` (int) instead of the router's, with the parameter ``vocab_size``."""
 
     graph_safe = True
 
@@ -41,7 +47,13 @@ class RoutedExperts(FeedForward):
         self.hidden = int(p["hidden_size"])
         self.inter = int(p["intermediate_size"])
         self.experts, self.top = int(p["experts"]), int(p["top"])
-        self.limit, self.alpha = float(p["limit"]), float(p["alpha"])
+        self.plain = p.get("limit") is None
+        # (the plain unit is the clamped one with no clamp, a slope of one and nothing added to the up half)
+        self.limit, self.alpha = (float("inf"), 1.0) if self.plain else (float(p["limit"]), float(p["alpha"]))
+        self.shift = 0.0 if self.plain else 1.0
+        self.tabled = p.get("router", "linear") == "table"
+        if p.get("router", "linear") not in ("linear", "table"):
+            raise ValueError(f"router {p['router']!r} is not one of linear, table")
         if not 0 < self.top <= self.experts:
             raise ValueError(f"a token cannot use {self.top} of {self.experts} experts")
         if not self.limit > 0:
@@ -60,7 +72,10 @@ class RoutedExperts(FeedForward):
         for i in range(e):
             out += [WeightSpec(f"{prefix}.e{i}.gate", (f, h)), WeightSpec(f"{prefix}.e{i}.up", (f, h)),
                     WeightSpec(f"{prefix}.e{i}.down", (h, f))]
-        out += [WeightSpec(f"{prefix}.router", (e, h)), WeightSpec(f"{prefix}.router.b", (e,), kind="vector")]
+        if p.get("router", "linear") == "table":
+            out.append(WeightSpec(f"{prefix}.table", (int(p["vocab_size"]), int(p["top"])), kind="int", init="distinct", free=e))
+        else:
+            out += [WeightSpec(f"{prefix}.router", (e, h)), WeightSpec(f"{prefix}.router.b", (e,), kind="vector")]
         if p.get("shared") is not None:
             out += part_class(p["shared"].kind).weight_specs(p["shared"], cls.join(prefix, "shared"))
         return out
@@ -73,9 +88,18 @@ class RoutedExperts(FeedForward):
             return rt.matrix(torch.stack(mats, dim=0))
 
         self.w_gate, self.w_up, self.w_down = stacked("gate"), stacked("up"), stacked("down")
-        self.w_router = rt.matrix(weights.get(f"{self.prefix}.router"))
-        self.b_router = rt.vector(weights.get(f"{self.prefix}.router.b"))
-        if self.top > rt.kernels.experts_max_top():
+        if self.tabled:
+            table = weights.get(f"{self.prefix}.table").to(torch.int32)
+            if int(table.min()) < 0 or int(table.max()) >= self.experts:
+                raise ValueError(f"{self.prefix}.table names experts outside [0, {self.experts})")
+            if self.top > 1 and bool((table.sort(dim=1).values.diff(dim=1) == 0).any()):
+                raise ValueError(f"{self.prefix}.table names an expert twice in a row")
+            self.table = table.to(rt.device).contiguous()
+            rt.kernels.experts_lib()
+        else:
+            self.w_router = rt.matrix(weights.get(f"{self.prefix}.router"))
+            self.b_router = rt.vector(weights.get(f"{self.prefix}.router.b"))
+        if not self.tabled and self.top > rt.kernels.experts_max_top():
             raise ValueError(f"{self.top} experts a token exceed the {rt.kernels.experts_max_top()} the routing kernel picks")
         if self.shared is not None:
             self.shared.load(weights, rt)
@@ -90,8 +114,6 @@ class RoutedExperts(FeedForward):
         rt = ctx.rt
         k = rt.kernels
         t, e, top = ctx.n_tokens, self.experts, self.top
-        logits = ctx.buf("experts.logits", (t, e), torch.float32)
-        k.gemm(x, self.w_router, logits, STORE_F32)
         rows = self.rows_a_tile(t, top, e)
         cap = k.experts_tile_capacity(t, e, top, rows)
         chosen = ctx.buf("experts.chosen", (t * top,), torch.int32)
@@ -99,12 +121,17 @@ class RoutedExperts(FeedForward):
         order = ctx.buf("experts.order", (t * top,), torch.int32)
         tiles = ctx.buf("experts.tiles", (4 * cap,), torch.int32)
         counts = ctx.buf("experts.counts", (e,), torch.int32)
-        k.experts_route(logits, self.b_router, top, rows, chosen, share, order, tiles, counts)
+        if self.tabled:
+            k.experts_route_table(ctx.token_ids, self.table, e, rows, chosen, share, order, tiles, counts)
+        else:
+            logits = ctx.buf("experts.logits", (t, e), torch.float32)
+            k.gemm(x, self.w_router, logits, STORE_F32)
+            k.experts_route(logits, self.b_router, top, rows, chosen, share, order, tiles, counts)
         slices = top + (1 if self.shared is not None else 0)
         partials = ctx.buf("experts.slices", (slices * t, self.hidden), torch.float32).view(slices, t, self.hidden)
         act = ctx.buf("experts.act", (t * top, self.inter), rt.dtype)
         k.experts_apply(x, self.w_gate, self.w_up, self.w_down, top, rows, order, tiles, share, self.limit, self.alpha,
-                        act, partials[:top])
+                        act, partials[:top], shift=self.shift)
         if self.shared is not None:
             self.shared.forward(ctx, x, partials[top], accumulate=False)
         pending = PendingAdd(partials)

@@ -11,7 +11,10 @@ from .base import Norm, WeightSpec, register_part
 @register_part("rmsnorm")
 class RMSNorm(Norm):
     """Parameters: ``size``, ``eps``; ``name`` overrides the tensor name.  With ``optional`` the
-    weight may be absent (a layer whose second half is missing never runs the norm)."""
+    weight may be absent (a layer whose second half is missing never runs the norm).  ``offset``
+    (default 0): the stored weight is the distance of the factor from this number, the row is
+    multiplied by ``offset + w`` (1 for weights stored around zero).  ``copies`` (default 1): the
+    stream holds that many copies ``[T, copies * size]`` and the norm reads their sum."""
 
     graph_safe = True
     repeatable = True
@@ -20,6 +23,8 @@ class RMSNorm(Norm):
         super().__init__(spec, prefix)
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
+        self.offset = float(spec.params.get("offset") or 0.0)
+        self.copies = int(spec.params.get("copies") or 1)
         self.weight = None
 
     @staticmethod
@@ -28,7 +33,8 @@ class RMSNorm(Norm):
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
-        return [WeightSpec(cls.tensor_name(spec, prefix), (int(spec["size"]),), kind="vector", init="norm",
+        return [WeightSpec(cls.tensor_name(spec, prefix), (int(spec["size"]),), kind="vector",
+                           init="around_zero" if spec.params.get("offset") else "norm",
                            optional=bool(spec.params.get("optional")))]
 
     def load(self, weights, rt) -> None:
@@ -36,9 +42,19 @@ class RMSNorm(Norm):
         if self.spec.params.get("optional") and name not in weights:
             return
         self.weight = rt.vector(weights.get(name))
+        if self.offset:
+            self.weight = self.weight + self.offset          # (float32: the factor as 32-bit arithmetic forms it)
 
     def forward(self, ctx, x, out, rows=None, pending=None) -> None:
         """``pending`` (a ``PendingAdd``): added to ``x`` first, in the same launch."""
+        if self.copies > 1 or hasattr(pending, "mix"):
+            # the sum of the copies, after what the last sublayer still has to write into them
+            if pending is not None and not hasattr(pending, "mix"):
+                raise ValueError("a stream of several copies takes the pending write of its own arrangement only")
+            ctx.rt.kernels.streams_step(x, self.copies, None if pending is None else pending.partials,
+                                        None if pending is None else pending.mix, None if pending is None else pending.gain,
+                                        None, self.weight, self.eps, out, rows)
+            return
         if pending is not None:
             ctx.rt.kernels.add_rmsnorm(x, pending.partials, self.weight, out, self.eps, rows)
         else:

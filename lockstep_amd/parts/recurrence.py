@@ -1,5 +1,6 @@
 """Linear-attention mixers that keep a matrix of fixed size per request and head instead of keys
-and values: one recurrence with a decay and a write gate for every row of the state,
+and values.  ``gated_delta`` (at the end of this file) is the delta rule with a decay a head and short
+convolutions in front; the two others share one recurrence with a decay and a write gate for every row of the state,
 
     S_t = diag(a_t) S_(t-1) + b_t v_t^T          S [dim, vdim] in float32, zero at the start
     o_t = S_t^T q_t
@@ -154,3 +155,90 @@ class Retention(_LinearRecurrence):
         gated = ctx.buf("recurrence.normed", (t, n * dv), rt.dtype)
         k.head_norm_gate(o, n, dv, None, raw[:, 2 * n * d + n * dv:], self.eps, gated)
         return project_out(ctx, gated, self.w_o, out, accumulate, defer, "recurrence.out_slices")
+
+
+@register_part("gated_delta")
+class GatedDelta(Mixer):
+    """The gated delta rule: a state matrix a head that forgets by a decay and is corrected, not
+    just added to, by every token:
+
+        S <- g_t S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
+
+    ``q = W_q h`` and ``k = W_k h`` (``num_kv_heads`` heads of ``head_dim``; head ``n`` of ``num_heads`` uses
+    q/k head ``n // (num_heads / num_kv_heads)``) and ``v = W_v h`` (``num_heads`` of ``value_dim``) pass a
+    short causal convolution a channel (``<tensor>.conv`` ``[channels, taps]``, the last column is the
+    current token's, zeros before the start) and SiLU; q and k are then unit vectors a head, ``x /
+    sqrt(sum x^2 + unit_eps)``, q also times ``head_dim^-1/2``.  ``beta = sigmoid(W_b h)``, ``g =
+    exp(-exp(A_log) softplus(W_a h + dt_bias))``, one of each a head.  Each head's ``o`` is divided by its
+    root mean square (``eps``), multiplied by ``norm [value_dim]`` and by ``silu(W_g h)``; then ``W_o``.
+
+    Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim``, ``value_dim``, ``taps``,
+    ``eps``, ``unit_eps``.  Tensors below the prefix: ``q``, ``k``, ``v`` with ``q.conv``, ``k.conv``,
+    ``v.conv``; ``b``, ``a`` ``[heads, hidden]``; ``A_log``, ``dt_bias`` ``[heads]``; ``g`` ``[heads*vdim,
+    hidden]``; ``norm`` ``[vdim]``; ``o``.
+
+    The projections are one matrix product stored in float32; convolutions, gates, the recurrence and
+    the per-head norm are computed in 32-bit.  A request's state slot holds the matrices and, behind
+    them, the last ``taps - 1`` inputs of every convolution channel."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        super().__init__(spec, prefix)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.heads, self.kv_heads = int(p["num_heads"]), int(p["num_kv_heads"])
+        self.d, self.dv, self.taps = int(p["head_dim"]), int(p["value_dim"]), int(p["taps"])
+        self.eps, self.unit_eps = float(p["eps"]), float(p["unit_eps"])
+        if min(self.heads, self.kv_heads, self.d, self.dv, self.taps) <= 0 or self.heads % self.kv_heads:
+            raise ValueError(f"{self.heads} heads over {self.kv_heads} query/key heads with sizes {self.d}, {self.dv} "
+                             f"and {self.taps} taps are not a gated delta mixer")
+        self.channels = 2 * self.kv_heads * self.d + self.heads * self.dv
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+
+    @classmethod
+    def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
+        p = spec.params
+        h, n, g, d, dv, m = (int(p[key]) for key in ("hidden_size", "num_heads", "num_kv_heads", "head_dim", "value_dim", "taps"))
+        return [WeightSpec(f"{prefix}.q", (g * d, h)), WeightSpec(f"{prefix}.q.conv", (g * d, m), kind="vector", init="unit"),
+                WeightSpec(f"{prefix}.k", (g * d, h)), WeightSpec(f"{prefix}.k.conv", (g * d, m), kind="vector", init="unit"),
+                WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.v.conv", (n * dv, m), kind="vector", init="unit"),
+                WeightSpec(f"{prefix}.b", (n, h)), WeightSpec(f"{prefix}.A_log", (n,), kind="vector"),
+                WeightSpec(f"{prefix}.norm", (dv,), kind="vector", init="norm"), WeightSpec(f"{prefix}.a", (n, h)),
+                WeightSpec(f"{prefix}.dt_bias", (n,), kind="vector"), WeightSpec(f"{prefix}.g", (n * dv, h)),
+                WeightSpec(f"{prefix}.o", (h, n * dv))]
+
+    def cache_spec(self):
+        return StateSpec((self.heads * self.d * self.dv + (self.taps - 1) * self.channels,), "float32")
+
+    def mixing_flops(self, tokens: int, start: int) -> float:
+        """Decay, two reads and a write of every state element per token."""
+        return 7.0 * self.heads * self.d * self.dv * tokens
+
+    def load(self, weights, rt) -> None:
+        if self.d > rt.kernels.delta_max_dim():
+            raise ValueError(f"a state of {self.d} rows a head is not supported: the delta rule kernel takes up to "
+                             f"{rt.kernels.delta_max_dim()}")
+        tensors = [weights.get(f"{self.prefix}.{n}") for n in ("q", "k", "v", "b", "a", "g")]
+        if len({t.dtype for t in tensors}) > 1:
+            tensors = [t.to(torch.float32) for t in tensors]
+        self.w_in = rt.matrix(torch.cat(tensors, dim=0))
+        self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
+        self.conv = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.conv").to(torch.float32) for n in "qkv"], dim=0))
+        self.a_log = rt.vector(weights.get(f"{self.prefix}.A_log"))
+        self.dt_bias = rt.vector(weights.get(f"{self.prefix}.dt_bias"))
+        self.norm = rt.vector(weights.get(f"{self.prefix}.norm"))
+        rt.kernels.mixers_lib()
+
+    def forward(self, ctx, run, x, out, accumulate: bool, defer: bool = False):
+        rt, k, t = ctx.rt, ctx.rt.kernels, ctx.n_tokens
+        n, g, d, dv = self.heads, self.kv_heads, self.d, self.dv
+        raw = ctx.buf("delta.in_f32", (t, self.w_in.shape[0]), torch.float32)
+        k.gemm(x, self.w_in, raw, STORE_F32)
+        o = ctx.buf("delta.o_f32", (t, n * dv), torch.float32)
+        scratch = ctx.buf("delta.scratch", (k.delta_scratch_floats(t, g, n, d, dv),), torch.float32)
+        k.delta_rule(raw, g, n, d, dv, self.conv, self.a_log, self.dt_bias, self.unit_eps, ctx.tok_seq, ctx.tok_pos,
+                     ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), scratch, o)
+        gated = ctx.buf("delta.normed", (t, n * dv), rt.dtype)
+        k.head_norm_gate(o, n, dv, self.norm, raw[:, self.channels + 2 * n:], self.eps, gated)
+        return project_out(ctx, gated, self.w_o, out, accumulate, defer, "delta.out_slices")

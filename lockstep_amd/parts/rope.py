@@ -125,6 +125,62 @@ class RotaryScaled(RotaryHalf):
         return list(range(0, self.rotary_dim, 2)) + list(range(1, self.rotary_dim, 2)) + list(range(self.rotary_dim, head_dim))
 
 
+@register_part("rope_ramped")
+class RotaryRamped(RotaryScaled):
+    """Rotary encoding whose frequencies are stretched along a ramp over the pair index, and whose cosines
+    and sines are enlarged.  Parameters: ``rotary_dim``, ``theta``, ``pairing`` and ``scaling`` (None, or
+    ``factor``, ``original``, ``fast``, ``slow``).  With ``c(t) = rotary_dim ln(original / (2 pi t)) / (2 ln
+    theta)``, the pair index at which a rotation makes ``t`` turns within ``original`` positions, ``lo =
+    max(floor(c(fast)), 0)`` and ``hi = min(ceil(c(slow)), rotary_dim - 1)``: pair ``i`` has the frequency
+    ``f_i / factor * r_i + f_i (1 - r_i)`` with ``r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``, and
+    both tables are multiplied by ``0.1 ln(factor) + 1``."""
+
+    def __init__(self, spec: PartSpec, prefix: str = ""):
+        scaling = spec.params.get("scaling")
+        super().__init__(PartSpec(spec.kind, {**spec.params, "scaling": None}), prefix)
+        self.spec = spec
+        self.ramp = None
+        if scaling:
+            self.ramp = tuple(float(scaling[key]) for key in ("factor", "original", "fast", "slow"))
+            factor, original, fast, slow = self.ramp
+            if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and self.theta > 1):
+                raise ValueError(f"a frequency ramp needs positive factor, original, fast and slow and theta > 1, got {scaling}")
+
+    def share_key(self):
+        return (self.rotary_dim, self.theta, "ramp", self.ramp)
+
+    def magnitude(self) -> float:
+        import math
+
+        return 1.0 if self.ramp is None else 0.1 * math.log(self.ramp[0]) + 1.0
+
+    def frequencies(self) -> torch.Tensor:
+        import math
+
+        half = self.rotary_dim // 2
+        index = torch.arange(0, half, dtype=torch.float64)
+        freq = 1.0 / (self.theta ** (index * 2.0 / self.rotary_dim))
+        if self.ramp is None:
+            return freq
+        factor, original, fast, slow = self.ramp
+
+        def pair_of(turns: float) -> float:
+            return self.rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo = max(math.floor(pair_of(fast)), 0)
+        hi = min(math.ceil(pair_of(slow)), self.rotary_dim - 1)
+        ramp = ((index - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        return freq / factor * ramp + freq * (1.0 - ramp)
+
+    def tables(self, positions: torch.Tensor):
+        angles = positions.to(torch.float64)[:, None] * self.frequencies()[None, :]
+        scale = self.magnitude()
+        return (angles.cos() * scale).to(torch.float32), (angles.sin() * scale).to(torch.float32)
+
+    def bind(self, rt) -> None:
+        self._store = _TABLES.setdefault((self.rotary_dim, self.theta, "ramp", self.ramp, str(rt.device)), [None, None])
+
+
 @register_part("no_position")
 class NoPosition(PositionEncoding):
     """Leaves queries and keys as they are."""

@@ -63,7 +63,7 @@ class SinkAttention(Mixer):
     ``value_dim``, ``position`` (a position-encoding ``PartSpec``), ``scale``, ``window`` / ``chunk``
     (None or a size; at most one of them), ``sink`` (None, ``"zero"`` or ``"learned"``), ``gate``,
     ``bias`` (biases of q, k, v), ``out_bias``, ``qk_norm`` (None or the eps of a norm over the whole
-    projection), ``shared_kv`` (the values are the keys as projected), ``distance_bias`` (None or
+    projection), ``head_norm`` (None or the eps of a norm without weights over every head of q and of k), ``shared_kv`` (the values are the keys as projected), ``distance_bias`` (None or
     ``{"farthest": D, "rows": B}``; ``rows`` only sizes random weights, a checkpoint's table says it itself).
     Tensors below the prefix: ``q``, ``k``, ``v``, ``o``; ``g`` (gate); ``q.b``, ``k.b``, ``v.b``;
     ``o.b``; ``q.norm``, ``k.norm``; ``rel [B, H]``; ``sink [H]``."""
@@ -85,6 +85,9 @@ class SinkAttention(Mixer):
         self.bias = bool(p.get("bias"))
         self.out_bias = bool(p.get("out_bias"))
         self.qk_norm = None if p.get("qk_norm") is None else float(p["qk_norm"])
+        self.head_norm = None if p.get("head_norm") is None else float(p["head_norm"])
+        if self.qk_norm is not None and self.head_norm is not None:
+            raise ValueError("a norm over the whole projection and a norm over every head: at most one")
         self.shared_kv = bool(p.get("shared_kv"))
         self.distance_bias = p.get("distance_bias")
         if self.nq % self.nkv:
@@ -271,10 +274,10 @@ class SinkAttention(Mixer):
         raw = ctx.buf("sink.in_f32", (t, self.w_in.shape[0]), torch.float32)
         k.gemm(x, self.w_in, raw, STORE_F32)
         q = ctx.buf("sink.q", (t, nq * self.dk), rt.dtype)
-        k.qkv_post(raw, t, nq, nkv, d, dv, self.b_in, self.q_norm, self.k_norm, self.qk_norm or 0.0, self.position.cos,
+        k.qkv_post(raw, t, nq, nkv, d, dv, self.b_in, self.q_norm, self.k_norm, self.qk_norm or self.head_norm or 0.0, self.position.cos,
                    self.position.sin, self.position.rotary_dim, self.neighbours, ctx.max_position, ctx.tok_seq,
                    ctx.tok_pos, ctx.seqs, group.table, q, key_pages, value_pages, group.page_size,
-                   keys_are_values=self.shared_kv, key_pad=self.dk)
+                   keys_are_values=self.shared_kv, key_pad=self.dk, per_head=self.head_norm is not None)
         key = self._block_key()
         attn = ctx.buf("sink.out", (t, nq * dv), rt.dtype)
         n_items, n_folds, row_tiles = ctx.notes[key]

@@ -41,8 +41,14 @@ def random_tensors(config: ModelConfig, seed: int, std: float | None = None, nor
         gen = _generator(seed, w.name)
         if any(n == -1 for n in w.shape):      # a size the checkpoint decides: the spec's own choice here
             w = dataclasses.replace(w, shape=tuple(w.free if n == -1 else n for n in w.shape))
-        if w.kind == "int":
+        if w.kind == "int" and w.init == "distinct":
+            # every row names w.shape[-1] different numbers below w.free
+            rows = [torch.randperm(w.free, generator=gen)[: w.shape[-1]] for _ in range(int(torch.tensor(w.shape[:-1]).prod()))]
+            value = torch.stack(rows).reshape(w.shape).to(torch.int32)
+        elif w.kind == "int":
             value = torch.zeros(w.shape, dtype=torch.int32)
+        elif w.init == "around_zero":
+            value = torch.randn(w.shape, generator=gen, dtype=torch.float32) * norm_std
         elif w.init == "norm":
             value = torch.ones(w.shape, dtype=torch.float32)
             if norm_std:
