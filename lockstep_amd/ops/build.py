@@ -8,7 +8,9 @@ Two kinds of library exist:
 ``attention<D>``    the attention kernels for one head size ``D``; a model
                     needs only its own;
 ``mixers``          Dynamic Tanh norm, clamped gated unit, soft cap, the linear
-                    recurrence with per-row gates and what surrounds it;
+                    recurrence with per-row gates and what surrounds it; the step of
+                    a residual stream of several copies, the passes around attention
+                    over a latent, a product a head, the gated delta rule;
 ``talking<shape>``  attention whose heads' scores are mixed before the softmax,
                     for one shape (query heads, kv heads, key and value size).
 ``sink<D>x<DV>``    grouped-query attention with a sink in the softmax, windows or
@@ -253,7 +255,8 @@ MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the 
 #: (query heads, kv heads, key size, value size) of the talking-heads attention the tests and measurements use
 DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
 #: (key size, value size) of the sink attention the tests and measurements use
-DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (24, 6), (128, 128))
+DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (24, 6), (128, 128),
+                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (192, 128))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,
