@@ -36,7 +36,9 @@ context lengths of ``--contexts`` (default 4,096, 8,192 and 16,384 tokens).
 
 measures the Bikovik design (talking-heads attention over a window that keeps the first tokens,
 HGRN2 and retention layers, Dynamic Tanh norms, a clamped gated feed-forward) and the Biberax
-design (chunked and biased attention with a sink and an output gate, routed experts; ``--designs``
+design (chunked and biased attention with a sink and an output gate, routed experts) or, with
+``--designs qwen3,toripel``, the Toripel design (a residual stream of four copies, the gated delta rule, windowed
+attention, attention over a cached latent, experts named by a table; ``--designs``
 chooses) beside the Qwen3 decoder at the same layer sizes (width, feed-forward, heads, head size, layers, vocabulary), both
 with random weights: prefill of one prompt and decode steps at batch 1 and 8, each with its
 fraction of the roofline.
@@ -91,7 +93,7 @@ class Workload:
         for layer_spec, layer in zip(spec.layers, model.layers):
             tensors = part_class(layer_spec.arrangement.kind).weight_specs(layer_spec)
             matrices = sum(_numel(w.shape) for w in tensors if w.kind == "matrix")
-            vectors = sum(_numel(w.shape) for w in tensors if w.kind != "matrix")
+            vectors = sum(_numel(w.shape) for w in tensors if w.kind not in ("matrix", "int"))   # (of a table a step reads a row a token)
             # a feed-forward of routed experts: a token multiplies with `top` of them, a step reads those it uses
             ff = getattr(layer, "feed_forward", None)
             routed = None
@@ -387,6 +389,38 @@ def biberax_like(qwen, layers: int, chunk: int = 8192, experts: int = 32, top: i
                              "norm": {"eps": qwen.rms_norm_eps}, "layers": [cycle[i % 4] for i in range(layers)]})
 
 
+def toripel_like(qwen, layers: int, window: int = 4096, experts: int = 32, top: int = 4, streams: int = 4):
+    """A Toripel configuration at the layer sizes of the Qwen3 configuration ``qwen``: a residual stream of four
+    copies; the layers cycle through the gated delta rule, windowed attention, attention over a latent, and
+    attention over the same latent read from the layer before; every mixer has the heads and head size of the
+    Qwen3 attention (the latent: as many elements as a head, half as many rotated ones beside it; the query
+    latent three times that).  A token's feed-forward multiplies with as many weights as the dense one: ``top``
+    experts, which a table names, of ``1 / top`` of the dense size each."""
+    from lockstep_amd.config import config_from_dict
+
+    heads, kv, d = qwen.num_attention_heads, qwen.num_key_value_heads, qwen.head_dim
+    moe = {"kind": "moe", "expert": {"ff": qwen.intermediate_size // top}, "router": {"experts": experts, "top": top}}
+    delta = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4}
+    windowed = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": window}}
+    over_latent = {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": 3 * d, "kv_rank": d, "scale": (d + d // 2) ** -0.5,
+                   "mask": {"size": window},
+                   "rot": {"dims": d // 2, "base": qwen.rope_theta,
+                           "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            out.append({"type": "delta", "mixer": delta, "mlp": moe})
+        elif kind == 1:
+            out.append({"type": "attention", "mixer": windowed, "mlp": moe})
+        elif kind == 2:
+            out.append({"type": "latent_attention", "mixer": over_latent, "mlp": moe})
+        else:
+            out.append({"type": "latent_attention", "mixer": dict(over_latent, kv_from=i - 1), "mlp": moe})
+    return config_from_dict({"architecture": "Toripel", "vocab": qwen.vocab_size, "width": qwen.hidden_size,
+                             "embedding": {"scale": 1.0}, "norm": {"eps": qwen.rms_norm_eps}, "streams": streams, "layers": out})
+
+
 def designs_record(args) -> dict:
     """Prefill and decode of the other designs beside Qwen3 at equal layer sizes."""
     import gc
@@ -404,7 +438,8 @@ def designs_record(args) -> dict:
     out = {"workload": "designs", "sizes": args.model, "layers": layers, "dtype": args.dtype,
            "prefill_tokens": args.prefill_len, "prompt_len": args.prompt_len, "steps": args.steps,
            "data": "synthetic: uniform random token ids, random weights", "designs": {}}
-    makers = {"qwen3": lambda: qwen, "bikovik": lambda: bikovik_like(qwen, layers), "biberax": lambda: biberax_like(qwen, layers)}
+    makers = {"qwen3": lambda: qwen, "bikovik": lambda: bikovik_like(qwen, layers), "biberax": lambda: biberax_like(qwen, layers),
+              "toripel": lambda: toripel_like(qwen, layers)}
     for name in args.designs.split(","):
         if name not in makers:
             raise SystemExit(f"--designs: {name!r} is not one of {', '.join(makers)}")
@@ -579,7 +614,7 @@ def main(argv=None) -> int:
                         "scheduler; contexts: prefill and decode at the context lengths of --contexts; designs: "
                         "the Bikovik and Biberax designs beside Qwen3 at the layer sizes of --model")
     p.add_argument("--contexts", default="4096,8192,16384", help="contexts: the context lengths, comma separated")
-    p.add_argument("--designs", default="qwen3,bikovik,biberax", help="designs: which of qwen3, bikovik, biberax, comma separated")
+    p.add_argument("--designs", default="qwen3,bikovik,biberax", help="designs: which of qwen3, bikovik, biberax, toripel, comma separated")
     p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
     p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")

@@ -365,6 +365,8 @@ def test_keys_just_inside_and_just_outside_a_window(tmp_path, kind, dtype, page)
 
     raw = _edge_case(kind)
     tensors = make_tensors(raw, seed=21, spread=1.5)
+    # (sinks that weigh as much as a row's best keys: a lost one moves the logits by half their size)
+    tensors = {name: (t.float() + 2.0).to(t.dtype) if name.endswith(".sink") else t for name, t in tensors.items()}
     model = load_model(write_model(tmp_path / "m", raw, tensors), dtype=dtype)
     oracle = plain.PlainToripel(raw, tensors)
     tokens = random_tokens(90, raw["vocab"], seed=6)
