@@ -17,20 +17,23 @@ __device__ int ls_mutants_dev = 0;  // external linkage: the compiler must not a
 namespace ls {
 
 // ---------------------------------------------------------------------------
-// Embedding: h[t, :] = float(E[token[t], :]) * scale.  A token id outside the table
+// Embedding: h[t, :] = float(E[token[t], :]) * scale, written `copies` times side by side.  A token id outside the table
 // writes zeros (the host rejects such ids before the launch; the kernel must
 // not fault on them).
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
                                                     float* __restrict__ out, int vocab, int width, long ld_out,
-                                                    float scale) {
+                                                    float scale, int copies) {
   const int t = blockIdx.x;
   const int id = tokens[t];
   const bool ok = id >= 0 && id < vocab;
   const T* row = table + (long)(ok ? id : 0) * width;
   float* dst = out + (long)t * ld_out;
-  for (int e = threadIdx.x; e < width; e += blockDim.x) dst[e] = ok ? to_f32(row[e]) * scale : 0.f;
+  for (int e = threadIdx.x; e < width; e += blockDim.x) {
+    const float v = ok ? to_f32(row[e]) * scale : 0.f;
+    for (int c = 0; c < copies; ++c) dst[(long)c * width + e] = v;   // (a stream of several copies starts with equal ones)
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -528,15 +531,15 @@ LS_DEFINE_MUTANT_API
 using namespace ls;
 
 extern "C" int ls_embed(int dtype, const int* tokens, const void* table, float* out, int n_tokens, int vocab,
-                        int width, long ld_out, float scale, void* stream) {
-  LS_REQUIRE(n_tokens > 0 && vocab > 0 && width > 0 && ld_out >= width, "embed: bad sizes");
+                        int width, long ld_out, float scale, int copies, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && vocab > 0 && width > 0 && copies > 0 && ld_out >= (long)copies * width, "embed: bad sizes");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (dtype == kF32)
     hipLaunchKernelGGL(embed_kernel<float>, dim3(n_tokens), dim3(256), 0, s, tokens, (const float*)table, out, vocab,
-                       width, ld_out, scale);
+                       width, ld_out, scale, copies);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, s, tokens, (const bf16_t*)table, out,
-                       vocab, width, ld_out, scale);
+                       vocab, width, ld_out, scale, copies);
   else
     return fail("embed: unknown dtype %d", dtype);
   return check_launch("embed");

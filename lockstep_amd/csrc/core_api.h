@@ -13,9 +13,9 @@ extern "C" {
 
 const char* ls_last_error();
 
-// Rows of the residual stream.  (embed: out = table[token] * scale)
+// Rows of the residual stream.  (embed: out = table[token] * scale, `copies` times side by side)
 int ls_embed(int dtype, const int* tokens, const void* table, float* out, int n_tokens, int vocab, int width,
-             long ld_out, float scale, void* stream);
+             long ld_out, float scale, int copies, void* stream);
 int ls_rmsnorm(int dtype, const float* x, const float* weight, void* out, const int* rows, int n_rows, int width,
                long ldx, long ld_out, float eps, void* stream);
 int ls_add_rmsnorm(int dtype, float* h, const float* P, int slices, int p_rows, const float* weight, void* out,

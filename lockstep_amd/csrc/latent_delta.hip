@@ -43,11 +43,20 @@ __device__ __forceinline__ float block_sum4(float v, float* scratch) {
 //           X'_t = sum_s mix[s][t] X_s + gain[t] y      for all t at once from the old copies
 //   read:   u = sum_t take[t] X'_t   (take == null: the plain sum of the copies)
 //           out = u / sqrt(mean(u^2) + eps) * weight     (T)
-// Thread t of 256 owns the elements 1024 c + 4 t + {0..3}; the sum of squares adds them in ascending order, then
+// Thread t of 256 owns the elements 1024 c + 4 t + {0..3}, c ascending; the sum of squares adds them in that order, then
 // a butterfly over the wave and the wave sums in wave order.  `row` = rows[r] when a row list is given.
 // ---------------------------------------------------------------------------
 constexpr int kMaxStreams = 8;
-constexpr int kStreamChunks = 8;  // a row of up to 1024 * kStreamChunks elements keeps its u in registers
+constexpr int kStreamChunks = 12;  // a row of up to 1024 * kStreamChunks elements keeps what it read in LDS
+
+__device__ __forceinline__ f32x4 load4(const float* __restrict__ p, int e, int W, bool vec_ok) {
+  if (vec_ok) return *reinterpret_cast<const f32x4*>(p + e);
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (e + i < W) v[i] = p[e + i];
+  return v;
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X, long ldx, int n, int W,
@@ -66,54 +75,65 @@ __global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X
   }
   __syncthreads();
   float* x = X + row * ldx;
-  float u[kStreamChunks][4];
+  // rows of whole vectors of four: a copy's elements and a slice's move as 16 bytes, all requested together
+  const bool vec_ok = W % 4 == 0 && ldx % 4 == 0;
+  extern __shared__ float u_s[];   // what the row's read gave, until the row's sum of squares is known (a thread's own elements)
   float part = 0.f;
+#pragma unroll 1
+  for (int e = 4 * (int)threadIdx.x; e < W; e += 1024) {
+    f32x4 copy[kMaxStreams];
 #pragma unroll
-  for (int c = 0; c < kStreamChunks; ++c) {
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < n) copy[s] = load4(x + (long)s * W, e, W, vec_ok);
+    if (P) {
+      const float* p = P + row * W;
+      f32x4 y = {0.f, 0.f, 0.f, 0.f};
+      int s = 0;
+      for (; s + 4 <= slices; s += 4) {
+        const f32x4 p0 = load4(p + s * p_stride, e, W, vec_ok), p1 = load4(p + (s + 1) * p_stride, e, W, vec_ok),
+                    p2 = load4(p + (s + 2) * p_stride, e, W, vec_ok), p3 = load4(p + (s + 3) * p_stride, e, W, vec_ok);
+        y = (((y + p0) + p1) + p2) + p3;
+      }
+      for (; s < slices; ++s) y = y + load4(p + s * p_stride, e, W, vec_ok);
+      f32x4 fresh[kMaxStreams];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = 1024 * c + 4 * (int)threadIdx.x + i;
-      u[c][i] = 0.f;
-      if (e >= W) continue;
-      float copy[kMaxStreams];
+      for (int t = 0; t < kMaxStreams; ++t) {
+        if (t >= n) continue;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s) copy[s] = s < n ? x[(long)s * W + e] : 0.f;
-      if (P) {
-        const float* p = P + row * W + e;
-        float y = 0.f;
-        for (int s = 0; s < slices; ++s) y = y + p[s * p_stride];
-        float fresh[kMaxStreams];
+        for (int s2 = 0; s2 < kMaxStreams; ++s2)
+          if (s2 < n) v = v + mix_s[s2 * n + t] * copy[s2];
+        fresh[t] = v + gain_s[t] * y;
+      }
 #pragma unroll
-        for (int t = 0; t < kMaxStreams; ++t) {
-          float v = 0.f;
+      for (int t = 0; t < kMaxStreams; ++t) {
+        if (t >= n) continue;
+        copy[t] = fresh[t];
+        if (vec_ok) {
+          *reinterpret_cast<f32x4*>(x + (long)t * W + e) = fresh[t];
+        } else {
 #pragma unroll
-          for (int s = 0; s < kMaxStreams; ++s)
-            if (s < n && t < n) v = v + mix_s[s * n + t] * copy[s];
-          fresh[t] = t < n ? v + gain_s[t] * y : 0.f;
-        }
-#pragma unroll
-        for (int t = 0; t < kMaxStreams; ++t) {
-          copy[t] = fresh[t];
-          if (t < n) x[(long)t * W + e] = fresh[t];
+          for (int i = 0; i < 4; ++i)
+            if (e + i < W) x[(long)t * W + e + i] = fresh[t][i];
         }
       }
-      float sum = 0.f;
-#pragma unroll
-      for (int t = 0; t < kMaxStreams; ++t)
-        if (t < n) sum = sum + take_s[t] * copy[t];
-      u[c][i] = sum;
-      part = part + sum * sum;
     }
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < kMaxStreams; ++t)
+      if (t < n) sum = sum + take_s[t] * copy[t];
+    if (out) *reinterpret_cast<f32x4*>(u_s + e) = sum;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part = part + sum[i] * sum[i];   // (elements beyond W are zeros)
   }
   if (!out) return;
   const float scale = 1.0f / sqrtf(block_sum4(part, scratch) / (float)W + eps);
+#pragma unroll 1
+  for (int e0 = 4 * (int)threadIdx.x; e0 < W; e0 += 1024) {
+    const f32x4 u = *reinterpret_cast<const f32x4*>(u_s + e0);
 #pragma unroll
-  for (int c = 0; c < kStreamChunks; ++c) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = 1024 * c + 4 * (int)threadIdx.x + i;
-      if (e < W) out[(long)r_out * ld_out + e] = from_f32<T>((u[c][i] * scale) * weight[e]);
-    }
+    for (int i = 0; i < 4; ++i)
+      if (e0 + i < W) out[(long)r_out * ld_out + e0 + i] = from_f32<T>((u[i] * scale) * weight[e0 + i]);
   }
 }
 
@@ -275,12 +295,12 @@ __global__ __launch_bounds__(256) void heads_product_kernel(const T* __restrict_
 //     butterfly), the query also times D^(-1/2).  Gates of head h: beta = sigmoid(b_h),
 //     decay = exp(-exp(A_log_h) softplus(a_h + dt_bias_h)).
 //     qk [T][2 G][dp] (queries, then keys; zeros beyond D), vv [T][H * DV], gates [T][H][2].
-// (2) delta_rule: a wave a (request, head, 16 columns of the state); lane (column lane / 4, quarter lane % 4)
-//     keeps the rows quarter * R + {0 .. R-1} of its column.  Per token, in order:
+// (2) delta_rule: a wave a (request, head, 64 / L columns of the state); L neighbouring lanes share a column, lane
+//     part p of them keeps the rows p * R + {0 .. R-1}.  Per token, in order:
 //       kS = decay * sum_r S[r] k[r];  u = beta (v - kS);  S[r] = decay S[r] + k[r] u;  o = sum_r S[r] q[r]
-//     (the sums: a lane's rows ascending by fused multiply-adds, then the quarters by exchanges inside the quad; the
+//     (the sums: a lane's rows in four interleaved chains of fused multiply-adds, then the lanes of a column by moves inside their row of sixteen; the
 //     decay multiplies the sum of the old state with the key, which is the decayed state's sum up to rounding).
-//     The operands of the next token are requested before a token is worked on.
+//     The operands of the token after next are requested before a token is worked on.
 // (3) delta_conv_state: the last M - 1 inputs of every channel become the state of the next step.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void delta_prep_kernel(
@@ -334,25 +354,32 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
   for (int i = lane; i < dp; i += 64) dst[i] = i < size ? channel(c0 + i) * scale : 0.f;
 }
 
-__device__ __forceinline__ float quad4_sum(float v) {
+// Sum over the L (4, 8 or 16) neighbouring lanes that share a column, by data-parallel moves inside a row of sixteen
+// lanes (no LDS): pairs, pairs of pairs, then the mirror image of the half row and of the row.  After every step
+// the lanes that were added hold the same value, so all L lanes end with the same bits.
+template <int L>
+__device__ __forceinline__ float lanes_sum(float v) {
   v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));  // lanes 1 0 3 2
   v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));  // lanes 2 3 0 1
+  if constexpr (L >= 8) v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));  // 7 - i
+  if constexpr (L >= 16) v = v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));  // 15 - i
   return v;
 }
 
-template <int R>
+// R rows a lane, L lanes a column (R * L rows, the head size rounded up), 64 / L columns a wave.
+template <int R, int L>
 __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict__ qk, const float* __restrict__ vv,
                                                         const float* __restrict__ gates, int G, int H, int D, int DV,
                                                         const SeqMeta* __restrict__ seqs, float* __restrict__ state,
                                                         long state_stride, float* __restrict__ out, long ldo) {
-  constexpr int dp = 4 * R;
+  constexpr int dp = L * R, COLS = 64 / L;
   const int seq = blockIdx.x / H, head = blockIdx.x % H;
   const SeqMeta m = seqs[seq];
   if (m.q_len <= 0) return;
-  const int lane = threadIdx.x, l16 = lane >> 2, quarter = lane & 3;
-  const int col = blockIdx.y * 16 + l16;
+  const int lane = threadIdx.x, lc = lane / L, part = lane % L;
+  const int col = blockIdx.y * COLS + lc;
   const bool col_ok = col < DV;
-  const int row0 = quarter * R;
+  const int row0 = part * R;
   const int kh = head / (H / G);
   float* mine = state + (long)m.table_row * state_stride + (long)head * D * DV;
   float S[R];
@@ -376,23 +403,26 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
     x.decay = gates[((long)t * H + head) * 2 + 1];
     return x;
   };
-  Operands next = fetch(m.q_off);
+  // the operands of the token after next are requested before a token is worked on
+  Operands next = fetch(m.q_off), after = m.q_len > 1 ? fetch(m.q_off + 1) : next;
   for (int i = 0; i < m.q_len; ++i) {
     const Operands now = next;
-    if (i + 1 < m.q_len) next = fetch(m.q_off + i + 1);
-    float ks = 0.f;
+    next = after;
+    if (i + 2 < m.q_len) after = fetch(m.q_off + i + 2);
+    // a lane's rows in four interleaved chains (rows r, r + 4, ... of each), added as (0 + 1) + (2 + 3)
+    float ks4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int r = 0; r < R; ++r) ks = fmaf(S[r], now.k[r >> 2][r & 3], ks);
-    ks = quad4_sum(ks) * now.decay;
+    for (int r = 0; r < R; ++r) ks4[r & 3] = fmaf(S[r], now.k[r >> 2][r & 3], ks4[r & 3]);
+    const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * now.decay;
     const float u = now.beta * (now.v - ks);
-    float o = 0.f;
+    float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       S[r] = fmaf(now.k[r >> 2][r & 3], u, now.decay * S[r]);
-      o = fmaf(S[r], now.q[r >> 2][r & 3], o);
+      o4[r & 3] = fmaf(S[r], now.q[r >> 2][r & 3], o4[r & 3]);
     }
-    o = quad4_sum(o);
-    if (quarter == 0 && col_ok) out[(long)(m.q_off + i) * ldo + head * DV + col] = o;
+    const float o = lanes_sum<L>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+    if (part == 0 && col_ok) out[(long)(m.q_off + i) * ldo + head * DV + col] = o;
   }
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -433,7 +463,7 @@ extern "C" int ls_streams_step(int dtype, float* X, long ldx, int n, int width, 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const long p_stride = (long)p_rows * width;
 #define LS_STREAMS(T_)                                                                                               \
-  hipLaunchKernelGGL(streams_step_kernel<T_>, dim3(n_rows), dim3(256), 0, s, X, ldx, n, width, P, slices, p_stride, \
+  hipLaunchKernelGGL(streams_step_kernel<T_>, dim3(n_rows), dim3(256), out ? ((width + 3) / 4) * 16 : 0, s, X, ldx, n, width, P, slices, p_stride, \
                      mix, gain, take, weight, eps, (T_*)out, ld_out, rows)
   if (dtype == kF32)
     LS_STREAMS(float);
@@ -563,16 +593,15 @@ extern "C" int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int
   hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, raw, ld, n_tokens, G, H, D, DV,
                      dp, M, taps, a_log, dt_bias, unit_eps, tok_seq, tok_pos, (const SeqMeta*)seqs, state, state_stride,
                      conv_at, qk, vv, gates);
-  const dim3 grid(n_seqs * H, (DV + 15) / 16);
-#define LS_DELTA(R_)                                                                                                  \
-  hipLaunchKernelGGL(delta_rule_kernel<R_>, grid, dim3(64), 0, s, qk, vv, gates, G, H, D, DV, (const SeqMeta*)seqs, state, \
-                     state_stride, out, ldo)
+#define LS_DELTA(R_, L_)                                                                                              \
+  hipLaunchKernelGGL((delta_rule_kernel<R_, L_>), dim3(n_seqs * H, (DV * L_ + 63) / 64), dim3(64), 0, s, qk, vv, gates, G, H, \
+                     D, DV, (const SeqMeta*)seqs, state, state_stride, out, ldo)
   switch (dp) {
-    case 16: LS_DELTA(4); break;
-    case 32: LS_DELTA(8); break;
-    case 64: LS_DELTA(16); break;
-    case 128: LS_DELTA(32); break;
-    default: LS_DELTA(64); break;
+    case 16: LS_DELTA(4, 4); break;
+    case 32: LS_DELTA(8, 4); break;
+    case 64: LS_DELTA(8, 8); break;
+    case 128: LS_DELTA(8, 16); break;
+    default: LS_DELTA(16, 16); break;
   }
 #undef LS_DELTA
   if (M > 1)

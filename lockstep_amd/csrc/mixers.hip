@@ -197,8 +197,14 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
   const int nq = H * D, nk = G * D, nv = G * DV;
   float rq = 1.0f, rk = 1.0f;
   if (per_head) {
-    // a wave a head of q | k: lane i adds the squares of the elements i, i + 64, ... ascending, then a butterfly
-    for (int head = threadIdx.x >> 6; head < H + G; head += 4) {
+    // a wave a head of q | k: lane i adds the squares of the elements i, i + 64, ... ascending, then a butterfly.
+    // Where the workgroups of a token each write one run of 256 elements, a workgroup needs the heads of its run only.
+    int h_lo = 0, h_hi = H + G;
+    if ((long)gridDim.y * 256 >= (long)(H + G) * Dp + (long)G * DV) {
+      h_lo = min(H + G, (int)(blockIdx.y * 256 / Dp));
+      h_hi = min(H + G, (int)((blockIdx.y * 256 + 255) / Dp) + 1);
+    }
+    for (int head = h_lo + (threadIdx.x >> 6); head < h_hi; head += 4) {
       float part = 0.f;
       for (int i = threadIdx.x & 63; i < D; i += 64) {
         const float x = row[head * D + i] + (bias ? bias[head * D + i] : 0.f);

@@ -331,20 +331,20 @@ class Kernels:
             c_long(ld_out), c_float(eps), _stream()))
 
     # -- rows -------------------------------------------------------------------
-    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
-        """``out[t] = table[tokens[t]] * scale`` as float32 rows."""
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0, copies: int = 1) -> None:
+        """``out[t] = table[tokens[t]] * scale`` as float32 rows, ``copies`` times side by side."""
         if not (tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous()):
             raise KernelError("embed tokens must be a contiguous int32 vector on the GPU")
         _rows_ok(table, "embed table"); _rows_ok(out, "embed out")
         if not (table.is_contiguous() and table.dtype in DTYPE_CODE):
             raise KernelError("embed table must be contiguous float32/bfloat16")
-        if not (out.dtype == torch.float32 and out.shape == (tokens.shape[0], table.shape[1])):
-            raise KernelError(f"embed out must be float32 [{tokens.shape[0]},{table.shape[1]}]")
+        if not (copies >= 1 and out.dtype == torch.float32 and out.shape == (tokens.shape[0], copies * table.shape[1])):
+            raise KernelError(f"embed out must be float32 [{tokens.shape[0]},{copies * table.shape[1]}]")
         if tokens.shape[0] == 0:
             return
         self._launch(self.core, self.core.ls_embed, (
             c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(table), _ptr(out), c_int(tokens.shape[0]),
-            c_int(table.shape[0]), c_int(table.shape[1]), c_long(out.stride(0)), c_float(scale), _stream()))
+            c_int(table.shape[0]), c_int(table.shape[1]), c_long(out.stride(0)), c_float(scale), c_int(copies), _stream()))
 
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float,
                 rows: torch.Tensor | None = None) -> None:

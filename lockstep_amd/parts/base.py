@@ -289,12 +289,13 @@ def deferred_rows(ctx, k: int, n: int) -> int:
 def project_out(ctx, x, weight, out, accumulate: bool, defer: bool, name: str):
     """A mixer's output projection ``out (+)= x @ weight.T`` into the float32 stream.  With ``defer`` a
     small step leaves the product as the sums of its K slices for the next reader of the stream
-    (a ``PendingAdd`` is returned), which cuts the work over K as well; else None."""
+    (a ``PendingAdd`` is returned, and ``out`` is not touched whatever ``accumulate`` says: the slices are
+    the product), which cuts the work over K as well; else None."""
     from ..ops import ADD_F32, STORE_F32
 
     k = ctx.rt.kernels
     inner = weight.shape[1]
-    if defer and accumulate and 0 < ctx.n_tokens <= deferred_rows(ctx, inner, out.shape[1]):
+    if defer and 0 < ctx.n_tokens <= deferred_rows(ctx, inner, out.shape[1]):
         slices = k.gemm_slices_count(inner)
         partials = ctx.buf(name, (slices * ctx.n_tokens, out.shape[1]), __import__("torch").float32)
         partials = partials.view(slices, ctx.n_tokens, out.shape[1])

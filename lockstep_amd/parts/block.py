@@ -154,9 +154,6 @@ class HyperConnections(Arrangement):
 
     graph_safe = True
 
-    #: steps of at most this many tokens ask their sublayers for slice sums (the write adds them up)
-    SLICE_ROWS = 256
-
     def __init__(self, layer_spec, prefix: str = ""):
         super().__init__(layer_spec, build_part)
         p = layer_spec.arrangement.params
@@ -237,14 +234,10 @@ class HyperConnections(Arrangement):
 
         t = ctx.n_tokens
         y = ctx.buf(f"streams.y.{sublayer}", (t, width), torch.float32)
-        if defers and t <= self.SLICE_ROWS:
-            # (a part that does not leave its product as slice sums after all adds it to zeros)
-            y.zero_()
-            left = call(y, True, True)
-            if isinstance(left, PendingAdd):
-                return left.partials
-        else:
-            call(y, False, False)
+        # (a part that defers leaves slice sums and does not touch y; else it stores its output there)
+        left = call(y, False, True) if defers else call(y, False, False)
+        if isinstance(left, PendingAdd):
+            return left.partials
         return y.view(1, t, width)
 
     def forward(self, ctx, run, h, pending=None):

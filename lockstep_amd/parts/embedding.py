@@ -30,9 +30,7 @@ class TokenEmbedding(Part):
         self.table = rt.matrix(weights.get(self.spec["name"]), share_key=weights.source_name(self.spec["name"]))
 
     def forward(self, ctx, tokens, out) -> None:
-        width = self.table.shape[1]
-        for c in range(self.copies):
-            ctx.rt.kernels.embed(tokens, self.table, out[:, c * width:(c + 1) * width] if self.copies > 1 else out, self.scale)
+        ctx.rt.kernels.embed(tokens, self.table, out, self.scale, self.copies)
 
 
 @register_part("linear_head")

@@ -135,9 +135,9 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             self.shared.forward(ctx, x, partials[top], accumulate=False)
         pending = PendingAdd(partials)
+        if defer and t <= DEFER_ROWS and self.hidden % 4 == 0:
+            return pending                 # (the slices are the result: ``out`` is not touched)
         if not accumulate:
             out.zero_()
-        if defer and accumulate and t <= DEFER_ROWS and self.hidden % 4 == 0:
-            return pending
         pending.flush(ctx, out)
         return None
