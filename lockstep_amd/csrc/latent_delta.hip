@@ -58,56 +58,56 @@ __device__ __forceinline__ f32x4 load4(const float* __restrict__ p, int e, int W
   return v;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X, long ldx, int n, int W,
+// (N, the number of copies, is a template parameter: every copy's load stands in straight-line code, so all of a
+// thread's loads are on their way before the first is used)
+template <typename T, int N>
+__global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X, long ldx, int W,
                                                            const float* __restrict__ P, int slices, long p_stride,
                                                            const float* __restrict__ mix, const float* __restrict__ gain,
                                                            const float* __restrict__ take, const float* __restrict__ weight,
                                                            float eps, T* __restrict__ out, long ld_out,
                                                            const int* __restrict__ rows) {
-  __shared__ float mix_s[kMaxStreams * kMaxStreams], gain_s[kMaxStreams], take_s[kMaxStreams], scratch[4];
+  __shared__ float mix_s[N * N], gain_s[N], take_s[N], scratch[4];
   const int r_out = blockIdx.x;
   const long row = rows ? rows[r_out] : r_out;
-  if (threadIdx.x < n * n) mix_s[threadIdx.x] = P ? mix[threadIdx.x] : 0.f;
-  if (threadIdx.x < n) {
+  if (threadIdx.x < N * N) mix_s[threadIdx.x] = P ? mix[threadIdx.x] : 0.f;
+  if (threadIdx.x < N) {
     gain_s[threadIdx.x] = P ? gain[threadIdx.x] : 0.f;
     take_s[threadIdx.x] = take ? take[threadIdx.x] : 1.0f;
   }
   __syncthreads();
   float* x = X + row * ldx;
-  // rows of whole vectors of four: a copy's elements and a slice's move as 16 bytes, all requested together
+  // rows of whole vectors of four: a copy's elements and a slice's move as 16 bytes
   const bool vec_ok = W % 4 == 0 && ldx % 4 == 0;
   extern __shared__ float u_s[];   // what the row's read gave, until the row's sum of squares is known (a thread's own elements)
   float part = 0.f;
+  constexpr int BATCH = 8;         // slice sums requested together
 #pragma unroll 1
   for (int e = 4 * (int)threadIdx.x; e < W; e += 1024) {
-    f32x4 copy[kMaxStreams];
+    f32x4 copy[N];
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
-      if (s < n) copy[s] = load4(x + (long)s * W, e, W, vec_ok);
+    for (int s = 0; s < N; ++s) copy[s] = load4(x + (long)s * W, e, W, vec_ok);
     if (P) {
       const float* p = P + row * W;
       f32x4 y = {0.f, 0.f, 0.f, 0.f};
-      int s = 0;
-      for (; s + 4 <= slices; s += 4) {
-        const f32x4 p0 = load4(p + s * p_stride, e, W, vec_ok), p1 = load4(p + (s + 1) * p_stride, e, W, vec_ok),
-                    p2 = load4(p + (s + 2) * p_stride, e, W, vec_ok), p3 = load4(p + (s + 3) * p_stride, e, W, vec_ok);
-        y = (((y + p0) + p1) + p2) + p3;
-      }
-      for (; s < slices; ++s) y = y + load4(p + s * p_stride, e, W, vec_ok);
-      f32x4 fresh[kMaxStreams];
+      for (int s0 = 0; s0 < slices; s0 += BATCH) {
+        f32x4 got[BATCH];
 #pragma unroll
-      for (int t = 0; t < kMaxStreams; ++t) {
-        if (t >= n) continue;
+        for (int u = 0; u < BATCH; ++u) got[u] = load4(p + (long)min(s0 + u, slices - 1) * p_stride, e, W, vec_ok);   // (clamped: no branch between the loads)
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+          if (s0 + u < slices) y = y + got[u];
+      }
+      f32x4 fresh[N];
+#pragma unroll
+      for (int t = 0; t < N; ++t) {
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s2 = 0; s2 < kMaxStreams; ++s2)
-          if (s2 < n) v = v + mix_s[s2 * n + t] * copy[s2];
+        for (int s2 = 0; s2 < N; ++s2) v = v + mix_s[s2 * N + t] * copy[s2];
         fresh[t] = v + gain_s[t] * y;
       }
 #pragma unroll
-      for (int t = 0; t < kMaxStreams; ++t) {
-        if (t >= n) continue;
+      for (int t = 0; t < N; ++t) {
         copy[t] = fresh[t];
         if (vec_ok) {
           *reinterpret_cast<f32x4*>(x + (long)t * W + e) = fresh[t];
@@ -120,8 +120,7 @@ __global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X
     }
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < kMaxStreams; ++t)
-      if (t < n) sum = sum + take_s[t] * copy[t];
+    for (int t = 0; t < N; ++t) sum = sum + take_s[t] * copy[t];
     if (out) *reinterpret_cast<f32x4*>(u_s + e) = sum;
 #pragma unroll
     for (int i = 0; i < 4; ++i) part = part + sum[i] * sum[i];   // (elements beyond W are zeros)
@@ -131,9 +130,16 @@ __global__ __launch_bounds__(256) void streams_step_kernel(float* __restrict__ X
 #pragma unroll 1
   for (int e0 = 4 * (int)threadIdx.x; e0 < W; e0 += 1024) {
     const f32x4 u = *reinterpret_cast<const f32x4*>(u_s + e0);
+    if (vec_ok) {
+      const f32x4 w = *reinterpret_cast<const f32x4*>(weight + e0);
+      T* dst = out + (long)r_out * ld_out + e0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (e0 + i < W) out[(long)r_out * ld_out + e0 + i] = from_f32<T>((u[i] * scale) * weight[e0 + i]);
+      for (int i = 0; i < 4; ++i) dst[i] = from_f32<T>((u[i] * scale) * w[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (e0 + i < W) out[(long)r_out * ld_out + e0 + i] = from_f32<T>((u[i] * scale) * weight[e0 + i]);
+    }
   }
 }
 
@@ -300,7 +306,7 @@ __global__ __launch_bounds__(256) void heads_product_kernel(const T* __restrict_
 //       kS = decay * sum_r S[r] k[r];  u = beta (v - kS);  S[r] = decay S[r] + k[r] u;  o = sum_r S[r] q[r]
 //     (the sums: a lane's rows in four interleaved chains of fused multiply-adds, then the lanes of a column by moves inside their row of sixteen; the
 //     decay multiplies the sum of the old state with the key, which is the decayed state's sum up to rounding).
-//     The operands of the token after next are requested before a token is worked on.
+//     A token's operands are requested eight (four) tokens before it is worked on.
 // (3) delta_conv_state: the last M - 1 inputs of every channel become the state of the next step.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void delta_prep_kernel(
@@ -328,14 +334,15 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
   const bool is_v = unit >= 2 * G;
   const int size = is_v ? DV : D;
   const int c0 = is_v ? 2 * G * D + (unit - 2 * G) * DV : unit * D;
-  // channel c at this token: convolution over the last M inputs, then silu
+  // channel c at this token: convolution over the last M inputs, then silu.  An input's address is chosen (this
+  // step's rows, or the state), then loaded: no branch stands between the loads of the taps.
   auto channel = [&](int c) LS_INLINED {
     float y = 0.f;
     for (int a = 0; a < M; ++a) {
       const int p = pos - (M - 1) + a;
-      const float in = p >= m.q_start ? raw[(long)(m.q_off + p - m.q_start) * ld + c]
-                                      : old[(long)(p - m.q_start + M - 1) * C + c];
-      y = y + taps[(long)c * M + a] * in;
+      const float* src = p >= m.q_start ? raw + (long)(m.q_off + p - m.q_start) * ld + c
+                                        : old + (long)(p - m.q_start + M - 1) * C + c;
+      y = y + taps[(long)c * M + a] * *src;
     }
     return silu_f(y);
   };
@@ -343,15 +350,23 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
     for (int i = lane; i < size; i += 64) vv[(long)t * H * DV + (c0 - 2 * G * D) + i] = channel(c0 + i);
     return;
   }
+  // a head of up to 256 elements: a lane keeps its up to four in registers between the sum and the scaling
+  float mine[4];
   float part = 0.f;
-  for (int i = lane; i < size; i += 64) {
-    const float x = channel(c0 + i);
-    part = part + x * x;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    mine[j] = i < size ? channel(c0 + i) : 0.f;
+    part = part + mine[j] * mine[j];
   }
   float scale = 1.0f / sqrtf(wave_sum(part) + unit_eps);
   if (unit < G) scale = scale * (1.0f / sqrtf((float)D));
   float* dst = qk + ((long)t * 2 * G + unit) * dp;
-  for (int i = lane; i < dp; i += 64) dst[i] = i < size ? channel(c0 + i) * scale : 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int i = lane + 64 * j;
+    if (i < dp) dst[i] = mine[j] * scale;
+  }
 }
 
 // Sum over the L (4, 8 or 16) neighbouring lanes that share a column, by data-parallel moves inside a row of sixteen
@@ -403,26 +418,35 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
     x.decay = gates[((long)t * H + head) * 2 + 1];
     return x;
   };
-  // the operands of the token after next are requested before a token is worked on
-  Operands next = fetch(m.q_off), after = m.q_len > 1 ? fetch(m.q_off + 1) : next;
-  for (int i = 0; i < m.q_len; ++i) {
-    const Operands now = next;
-    next = after;
-    if (i + 2 < m.q_len) after = fetch(m.q_off + i + 2);
-    // a lane's rows in four interleaved chains (rows r, r + 4, ... of each), added as (0 + 1) + (2 + 3)
-    float ks4[4] = {0.f, 0.f, 0.f, 0.f};
+  // the operands of the token DEPTH tokens on are requested before a token is worked on (a ring of registers; the
+  // index is clamped to the request's last token, so no branch stands between the requests)
+  constexpr int DEPTH = R <= 8 ? 8 : 4;
+  const int last = m.q_off + m.q_len - 1;
+  Operands ring[DEPTH];
 #pragma unroll
-    for (int r = 0; r < R; ++r) ks4[r & 3] = fmaf(S[r], now.k[r >> 2][r & 3], ks4[r & 3]);
-    const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * now.decay;
-    const float u = now.beta * (now.v - ks);
-    float o4[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < DEPTH; ++j) ring[j] = fetch(min(m.q_off + j, last));
+  for (int i0 = 0; i0 < m.q_len; i0 += DEPTH) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      S[r] = fmaf(now.k[r >> 2][r & 3], u, now.decay * S[r]);
-      o4[r & 3] = fmaf(S[r], now.q[r >> 2][r & 3], o4[r & 3]);
+    for (int j = 0; j < DEPTH; ++j) {
+      const int i = i0 + j;
+      if (i >= m.q_len) break;
+      const Operands now = ring[j];
+      ring[j] = fetch(min(m.q_off + i + DEPTH, last));
+      // a lane's rows in four interleaved chains (rows r, r + 4, ... of each), added as (0 + 1) + (2 + 3)
+      float ks4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < R; ++r) ks4[r & 3] = fmaf(S[r], now.k[r >> 2][r & 3], ks4[r & 3]);
+      const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * now.decay;
+      const float u = now.beta * (now.v - ks);
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] = fmaf(now.k[r >> 2][r & 3], u, now.decay * S[r]);
+        o4[r & 3] = fmaf(S[r], now.q[r >> 2][r & 3], o4[r & 3]);
+      }
+      const float o = lanes_sum<L>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+      if (part == 0 && col_ok) out[(long)(m.q_off + i) * ldo + head * DV + col] = o;
     }
-    const float o = lanes_sum<L>((o4[0] + o4[1]) + (o4[2] + o4[3]));
-    if (part == 0 && col_ok) out[(long)(m.q_off + i) * ldo + head * DV + col] = o;
   }
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -462,15 +486,20 @@ extern "C" int ls_streams_step(int dtype, float* X, long ldx, int n, int width, 
   LS_REQUIRE(!out || (weight && ld_out >= width && eps > 0.f), "streams_step: a read needs a weight and eps");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const long p_stride = (long)p_rows * width;
-#define LS_STREAMS(T_)                                                                                               \
-  hipLaunchKernelGGL(streams_step_kernel<T_>, dim3(n_rows), dim3(256), out ? ((width + 3) / 4) * 16 : 0, s, X, ldx, n, width, P, slices, p_stride, \
-                     mix, gain, take, weight, eps, (T_*)out, ld_out, rows)
-  if (dtype == kF32)
-    LS_STREAMS(float);
-  else if (dtype == kBF16)
-    LS_STREAMS(bf16_t);
-  else
-    return fail("streams_step: unknown dtype %d", dtype);
+  LS_REQUIRE(dtype == kF32 || dtype == kBF16, "streams_step: unknown dtype %d", dtype);
+  const size_t lds = out ? (size_t)((width + 3) / 4) * 16 : 0;
+#define LS_STREAMS(N_)                                                                                               \
+  case N_:                                                                                                           \
+    if (dtype == kF32)                                                                                               \
+      hipLaunchKernelGGL((streams_step_kernel<float, N_>), dim3(n_rows), dim3(256), lds, s, X, ldx, width, P, slices, \
+                         p_stride, mix, gain, take, weight, eps, (float*)out, ld_out, rows);                         \
+    else                                                                                                             \
+      hipLaunchKernelGGL((streams_step_kernel<bf16_t, N_>), dim3(n_rows), dim3(256), lds, s, X, ldx, width, P, slices, \
+                         p_stride, mix, gain, take, weight, eps, (bf16_t*)out, ld_out, rows);                        \
+    break;
+  switch (n) {
+    LS_STREAMS(1) LS_STREAMS(2) LS_STREAMS(3) LS_STREAMS(4) LS_STREAMS(5) LS_STREAMS(6) LS_STREAMS(7) LS_STREAMS(8)
+  }
 #undef LS_STREAMS
   return check_launch("streams_step");
 }
