@@ -256,7 +256,7 @@ MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the 
 DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
 #: (key size, value size) of the sink attention the tests and measurements use
 DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (24, 6), (128, 128),
-                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (192, 128))
+                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (48, 32), (192, 128))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,

@@ -84,3 +84,20 @@ def test_init_writes_a_biberax_folder_from_its_preset(tmp_path):
         assert name in names, name
     assert "l1.mix.v" not in names and "l3.mlp.gate" not in names
     assert tuple(handle.shape("l1.mix.rel")) == (16, 4)
+
+
+def test_init_writes_a_toripel_folder_from_its_preset(tmp_path):
+    from lockstep_amd.config import ToripelConfig, config_from_dir
+    from lockstep_amd.weights import SafetensorsFile
+
+    done = run("init", "--preset", "toripel-tiny", "--out", str(tmp_path / "k"), "--seed", "2")
+    assert done.returncode == 0, done.stderr
+    config = config_from_dir(tmp_path / "k")
+    assert isinstance(config, ToripelConfig) and config.width == 128 and len(config.layers) == 4 and config.streams == 2
+    handle = SafetensorsFile(tmp_path / "k" / "model.safetensors")
+    names = handle.keys()
+    for name in ("embed", "head", "final.norm", "l0.mix.q.conv", "l0.mix.A_log", "l0.hc1.mix", "l0.hc2.in", "l0.mlp.table",
+                 "l0.mlp.e7.down", "l1.mix.k.b", "l2.mix.dkv", "l2.mix.dkv.norm", "l2.mix.sink", "l3.mix.uk", "l3.mix.dq.norm"):
+        assert name in names, name
+    assert "l3.mix.dkv" not in names and "l3.mlp.table" not in names and "l0.mlp.router" not in names
+    assert tuple(handle.shape("l0.mlp.table")) == (640, 2) and tuple(handle.shape("l2.mix.dkv")) == (48, 128)
