@@ -235,7 +235,7 @@ class HyperConnections(Arrangement):
         t = ctx.n_tokens
         y = ctx.buf(f"streams.y.{sublayer}", (t, width), torch.float32)
         # (a part that defers leaves slice sums and does not touch y; else it stores its output there)
-        left = call(y, False, True) if defers else call(y, False, False)
+        left = call(y, False, "any") if defers else call(y, False, False)
         if isinstance(left, PendingAdd):
             return left.partials
         return y.view(1, t, width)

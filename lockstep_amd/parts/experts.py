@@ -110,7 +110,9 @@ class RoutedExperts(FeedForward):
         each = n_tokens * top / experts
         return 16 if each <= 16 else 32 if each <= 64 else 64
 
-    def forward(self, ctx, x, out, accumulate: bool, defer: bool = False):
+    def forward(self, ctx, x, out, accumulate: bool, defer=False):
+        """``defer``: True leaves the slices to the next reader of the stream in steps of up to ``DEFER_ROWS`` tokens;
+        ``"any"`` in every step (a reader that takes slices of any number of rows)."""
         rt = ctx.rt
         k = rt.kernels
         t, e, top = ctx.n_tokens, self.experts, self.top
@@ -135,7 +137,7 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             self.shared.forward(ctx, x, partials[top], accumulate=False)
         pending = PendingAdd(partials)
-        if defer and t <= DEFER_ROWS and self.hidden % 4 == 0:
+        if defer and (defer == "any" or t <= DEFER_ROWS) and self.hidden % 4 == 0:
             return pending                 # (the slices are the result: ``out`` is not touched)
         if not accumulate:
             out.zero_()
