@@ -39,8 +39,8 @@
 namespace ls {
 
 constexpr int D = LS_SA_DIM, DV = LS_SA_VDIM;
-static_assert(D % 8 == 0 && D <= 256, "key size must be a multiple of 8 up to 256");
-static_assert(DV >= 1 && DV <= 256, "value size must be at most 256");
+static_assert(D % 8 == 0 && D <= 640, "key size must be a multiple of 8 up to 640");
+static_assert(DV >= 1 && DV <= 512, "value size must be at most 512");
 constexpr int VB = (DV + 15) / 16;  // blocks of 16 value columns (the last may be partial)
 constexpr int kTileKeys = 32;
 constexpr int kMaxWaves = 4;        // query heads of a key/value head that share a workgroup

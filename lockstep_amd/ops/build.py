@@ -228,8 +228,8 @@ def build_talking(heads: int, kv_heads: int, dim: int, vdim: int, force: bool = 
 
 def build_sink(dim: int, vdim: int, force: bool = False) -> Path:
     """The sink attention library of one key size and one value size."""
-    if dim % 8 or not 8 <= dim <= 256 or not 1 <= vdim <= 256:
-        raise BuildError(f"key size {dim} / value size {vdim} are not supported: a multiple of 8 up to 256 / at most 256")
+    if dim % 8 or not 8 <= dim <= 640 or not 1 <= vdim <= 512:
+        raise BuildError(f"key size {dim} / value size {vdim} are not supported: a multiple of 8 up to 640 / at most 512")
     return build(f"sink{dim}x{vdim}", SINK_SOURCES, (f"-DLS_SA_DIM={dim}", f"-DLS_SA_VDIM={vdim}"), force)
 
 
@@ -256,7 +256,7 @@ MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the 
 DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
 #: (key size, value size) of the sink attention the tests and measurements use
 DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (24, 6), (128, 128),
-                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (48, 32), (192, 128))
+                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (48, 32), (192, 128), (320, 256))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,

@@ -88,6 +88,9 @@ SINGLE = {
     "windowed": dict(page_size=8, raw=config(64, 96, [bare(windowed(4, 2, 32, 16, window=20, scale=0.5))], streams=2)),
     "latent": dict(page_size=8, raw=config(64, 96, [
         bare(latent(4, 16, 16, 24, q_rank=32, kv_rank=48, window=26, scale=0.25, scaling=(4.0, 32, 8.0, 1.0)))], streams=2)),
+    # a latent of 256 elements beside a shared key part of 64: a key head of 320 elements, values of 256
+    "latent_wide": dict(page_size=16, raw=config(64, 96, [
+        bare(latent(2, 16, 64, 16, q_rank=32, kv_rank=256, window=30, scale=0.1, dims=32))], streams=2)),
     "delta": dict(page_size=8, raw=config(64, 96, [bare(delta(4, 2, 32, 16, taps=4))], streams=2)),
     "tabled": dict(page_size=8, raw=config(64, 96, [tabled(windowed(2, 1, 16, 16, window=None, scale=0.5), 40, experts=7, top=3)],
                                            streams=4)),
