@@ -402,46 +402,59 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
   for (int r = 0; r < R; ++r) S[r] = (row0 + r < D && col_ok) ? mine[(long)(row0 + r) * DV + col] : 0.f;
   struct Operands {
     f32x4 q[R / 4], k[R / 4];
-    float v, beta, decay;
+    float v, gate;   // gate: beta in the even lanes, the decay in the odd ones
   };
-  auto fetch = [&](int t) LS_INLINED {
+  // Pointers to the operands of the token that is requested next; they move on by a token after every request and
+  // stay on the request's last token (no index arithmetic and no branch between the requests).  beta and the decay
+  // are fetched by the lanes (even: beta, odd: decay) and handed round inside the quad: a load whose address is
+  // the same in every lane would go through the scalar cache, whose loads return in any order, so that a wait for
+  // one of them waits for all, also for those of the tokens ahead.
+  const float* q_at = qk + ((long)m.q_off * 2 * G + kh) * dp + row0;
+  const float* k_at = q_at + (long)G * dp;
+  const float* v_at = vv + (long)m.q_off * H * DV + head * DV + (col_ok ? col : 0);
+  const float* g_at = gates + ((long)m.q_off * H + head) * 2 + (lane & 1);
+  int left = m.q_len - 1;   // tokens behind the one the pointers stand on
+  auto fetch = [&]() LS_INLINED {
     Operands x;
-    const float* q = qk + ((long)t * 2 * G + kh) * dp + row0;
-    const float* k = qk + ((long)t * 2 * G + G + kh) * dp + row0;
 #pragma unroll
     for (int j = 0; j < R / 4; ++j) {
-      x.q[j] = *reinterpret_cast<const f32x4*>(q + 4 * j);
-      x.k[j] = *reinterpret_cast<const f32x4*>(k + 4 * j);
+      x.q[j] = *reinterpret_cast<const f32x4*>(q_at + 4 * j);
+      x.k[j] = *reinterpret_cast<const f32x4*>(k_at + 4 * j);
     }
-    x.v = col_ok ? vv[(long)t * H * DV + head * DV + col] : 0.f;
-    x.beta = gates[((long)t * H + head) * 2];
-    x.decay = gates[((long)t * H + head) * 2 + 1];
+    x.v = *v_at;
+    x.gate = *g_at;
+    const long step = left > 0 ? 1 : 0;
+    left -= (int)step;
+    q_at += step * 2 * G * dp;
+    k_at += step * 2 * G * dp;
+    v_at += step * H * DV;
+    g_at += step * H * 2;
     return x;
   };
-  // the operands of the token DEPTH tokens on are requested before a token is worked on (a ring of registers; the
-  // index is clamped to the request's last token, so no branch stands between the requests)
+  // the operands of the token DEPTH tokens on are requested before a token is worked on (a ring of registers)
   constexpr int DEPTH = R <= 8 ? 8 : 4;
-  const int last = m.q_off + m.q_len - 1;
   Operands ring[DEPTH];
 #pragma unroll
-  for (int j = 0; j < DEPTH; ++j) ring[j] = fetch(min(m.q_off + j, last));
+  for (int j = 0; j < DEPTH; ++j) ring[j] = fetch();
   for (int i0 = 0; i0 < m.q_len; i0 += DEPTH) {
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) {
       const int i = i0 + j;
       if (i >= m.q_len) break;
       const Operands now = ring[j];
-      ring[j] = fetch(min(m.q_off + i + DEPTH, last));
+      ring[j] = fetch();
+      const float beta = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(now.gate), 0x00, 0xF, 0xF, true));   // lane 0 of the quad
+      const float decay = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(now.gate), 0x55, 0xF, 0xF, true));  // lane 1
       // a lane's rows in four interleaved chains (rows r, r + 4, ... of each), added as (0 + 1) + (2 + 3)
       float ks4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < R; ++r) ks4[r & 3] = fmaf(S[r], now.k[r >> 2][r & 3], ks4[r & 3]);
-      const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * now.decay;
-      const float u = now.beta * (now.v - ks);
+      const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * decay;
+      const float u = beta * (now.v - ks);
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        S[r] = fmaf(now.k[r >> 2][r & 3], u, now.decay * S[r]);
+        S[r] = fmaf(now.k[r >> 2][r & 3], u, decay * S[r]);
         o4[r & 3] = fmaf(S[r], now.q[r >> 2][r & 3], o4[r & 3]);
       }
       const float o = lanes_sum<L>((o4[0] + o4[1]) + (o4[2] + o4[3]));
