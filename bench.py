@@ -405,7 +405,7 @@ def toripel_like(qwen, layers: int, window: int = 4096, experts: int = 32, top: 
     over_latent = {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "q_rank": 3 * d, "kv_rank": d, "scale": (d + d // 2) ** -0.5,
                    "mask": {"size": window},
                    "rot": {"dims": d // 2, "base": qwen.rope_theta,
-                           "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+                           "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     out = []
     for i in range(layers):
         kind = i % 4
