@@ -137,7 +137,7 @@ class RoutedExperts(FeedForward):
         if self.shared is not None:
             self.shared.forward(ctx, x, partials[top], accumulate=False)
         pending = PendingAdd(partials)
-        if defer and (defer == "any" or t <= DEFER_ROWS) and self.hidden % 4 == 0:
+        if defer == "any" or (defer and t <= DEFER_ROWS and self.hidden % 4 == 0):
             return pending                 # (the slices are the result: ``out`` is not touched)
         if not accumulate:
             out.zero_()

@@ -265,7 +265,7 @@ def test_experts_that_a_table_names(dtype, tokens, experts, top, width, ff):
 # whole models
 # ---------------------------------------------------------------------------
 
-@pytest.mark.parametrize("kind", ["windowed", "latent", "latent_wide", "delta", "tabled"])
+@pytest.mark.parametrize("kind", ["windowed", "latent", "latent_wide", "delta", "tabled", "odd_width"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_each_mechanism_alone_whole_and_in_portions(models, kind, dtype):
     model, oracle, raw, page, _ = models(kind, dtype, table=SINGLE)

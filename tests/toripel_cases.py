@@ -92,6 +92,8 @@ SINGLE = {
     "latent_wide": dict(page_size=16, raw=config(64, 96, [
         bare(latent(2, 16, 64, 16, q_rank=32, kv_rank=256, window=30, scale=0.1, dims=32))], streams=2)),
     "delta": dict(page_size=8, raw=config(64, 96, [bare(delta(4, 2, 32, 16, taps=4))], streams=2)),
+    # a width that is no multiple of 4 (rows that do not move as vectors), three copies
+    "odd_width": dict(page_size=8, raw=config(90, 96, [tabled(delta(3, 1, 8, 8, taps=2), 20, experts=3, top=2)], streams=3)),
     "tabled": dict(page_size=8, raw=config(64, 96, [tabled(windowed(2, 1, 16, 16, window=None, scale=0.5), 40, experts=7, top=3)],
                                            streams=4)),
 }
