@@ -9,9 +9,10 @@ from .qwen3 import Qwen3Config
 from .bikovik import BikovikConfig
 from .biberax import BiberaxConfig
 from .toripel import ToripelConfig
+from .narurax import NaruraxConfig
 
 __all__ = [
     "ConfigError", "LayerSpec", "ModelConfig", "ModelSpec", "PartSpec", "ScheduleEntry",
     "config_class_for", "config_from_dict", "config_from_dir", "known_architectures",
-    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig", "BiberaxConfig", "ToripelConfig",
+    "register_architecture", "unregister_architecture", "Qwen3Config", "BikovikConfig", "BiberaxConfig", "ToripelConfig", "NaruraxConfig",
 ]

@@ -94,12 +94,15 @@ class ScheduleEntry:
     entries).  ``cache`` is the cache unit the mixer uses in this run; units
     are numbered by the model spec.  ``writes_cache`` is False when the run
     only reads a unit that another entry fills (sharing another layer's keys
-    and values).
+    and values).  ``state`` is a second unit, for what the layer's arrangement
+    itself keeps per request between steps (``Arrangement.state_spec``), or
+    None where it keeps nothing.
     """
 
     layer: int
     cache: int
     writes_cache: bool = True
+    state: int | None = None
 
 
 @dataclass(frozen=True)
@@ -119,9 +122,14 @@ class ModelSpec:
     #: several that an arrangement with hyper-connections reads and writes; the embedding fills them and the
     #: final norm reads their sum
     residual_copies: int = 1
+    #: the cache unit of what the embedding keeps per request between steps (``state_spec`` of its part), or None
+    embedding_state: int | None = None
 
     def cache_units(self) -> int:
-        return 1 + max((e.cache for e in self.schedule), default=-1)
+        units = [e.cache for e in self.schedule] + [e.state for e in self.schedule if e.state is not None]
+        if self.embedding_state is not None:
+            units.append(self.embedding_state)
+        return 1 + max(units, default=-1)
 
 
 @dataclass(frozen=True)

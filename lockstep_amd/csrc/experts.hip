@@ -35,8 +35,10 @@ __device__ __forceinline__ float sigmoid_e(float x) { return 1.0f / (1.0f + expf
 // ---------------------------------------------------------------------------
 constexpr int kMaxPerLane = 8;   // experts a lane holds: up to 512 experts
 
+// scoring 0: the weights are the softmax over the chosen logits; 1: each chosen expert weighs the sigmoid of its own
+// logit, and nothing is renormalised (the sigmoid grows with the logit, so the largest logits are the largest scores).
 __device__ __forceinline__ void pick_top(const float* __restrict__ row, const float* __restrict__ bias, int E, int top,
-                                         int lane, int* __restrict__ picked, float* __restrict__ share) {
+                                         int lane, int* __restrict__ picked, float* __restrict__ share, int scoring) {
   float mine[kMaxPerLane];
 #pragma unroll
   for (int m = 0; m < kMaxPerLane; ++m) {
@@ -76,7 +78,7 @@ __device__ __forceinline__ void pick_top(const float* __restrict__ row, const fl
   const float sum = wave_sum(ex);
   if (lane < top) {
     picked[lane] = my_pick;
-    share[lane] = ex / sum;
+    share[lane] = scoring == 1 ? sigmoid_e(my_value) : ex / sum;
   }
 }
 
@@ -93,10 +95,10 @@ __global__ __launch_bounds__(256) void route_table_kernel(const int* __restrict_
 
 __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ z, long ldz,
                                                          const float* __restrict__ bias, int n_tokens, int E, int top,
-                                                         int* __restrict__ expert, float* __restrict__ weight) {
+                                                         int* __restrict__ expert, float* __restrict__ weight, int scoring) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= n_tokens) return;
-  pick_top(z + (long)t * ldz, bias, E, top, threadIdx.x & 63, expert + (long)t * top, weight + (long)t * top);
+  pick_top(z + (long)t * ldz, bias, E, top, threadIdx.x & 63, expert + (long)t * top, weight + (long)t * top, scoring);
 }
 
 // ---------------------------------------------------------------------------
@@ -180,7 +182,8 @@ __global__ __launch_bounds__(1024) void route_small_kernel(const float* __restri
                                                            int rows_a_tile, int* __restrict__ expert,
                                                            float* __restrict__ weight, int* __restrict__ order,
                                                            int* __restrict__ tiles, int cap,
-                                                           const int* __restrict__ token_ids, const int* __restrict__ table) {
+                                                           const int* __restrict__ token_ids, const int* __restrict__ table,
+                                                           int scoring) {
   __shared__ int picks_s[kSmallPairs];
   __shared__ float share_s[16][kMaxTop];
   __shared__ int counts_s[kSmallExperts];
@@ -195,7 +198,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(const float* __restri
     }
   }
   for (int t = w; t < n_tokens && !table; t += 16) {
-    pick_top(z + (long)t * ldz, bias, E, top, lane, picks_s + t * top, share_s[w]);
+    pick_top(z + (long)t * ldz, bias, E, top, lane, picks_s + t * top, share_s[w], scoring);
     if (lane < top) {
       expert[(long)t * top + lane] = picks_s[t * top + lane];
       weight[(long)t * top + lane] = share_s[w][lane];
@@ -219,7 +222,9 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
                                                               const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                               int F, int K, int top, const int* __restrict__ order,
                                                               const int* __restrict__ tiles, float limit, float alpha, float shift,
-                                                              T* __restrict__ act, long ldy) {
+                                                              const float* __restrict__ in_weight, T* __restrict__ act, long ldy) {
+  // in_weight (or null): a pair's routing weight multiplies the expert's input, w * x, so both products are scaled
+  // by it before the gated unit (the down product then adds the expert's output as it is)
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
   const int e = tiles[4 * blockIdx.x];
   if (e < 0) return;
@@ -290,12 +295,13 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
   for (int r = 0; r < RT; ++r) {
     if (!x_ok[r]) continue;
     T* dst = act + (long)(first + 16 * r + l16) * ldy;
+    const float wt = in_weight ? in_weight[order[first + 16 * r + l16]] : 1.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = col0 + 4 * quad + i;
       if (c < F) {
-        const float g = fminf(acc_g[r][i], limit);
-        const float u = fminf(fmaxf(acc_u[r][i], -limit), limit);
+        const float g = fminf(acc_g[r][i] * wt, limit);
+        const float u = fminf(fmaxf(acc_u[r][i] * wt, -limit), limit);
         dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + shift));
       }
     }
@@ -366,7 +372,7 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
   for (int r = 0; r < RT; ++r) {
     if (!y_ok[r]) continue;
     const int pair = order[first + 16 * r + l16];
-    const float share = weight[pair];
+    const float share = weight ? weight[pair] : 1.0f;
     float* dst = P + ((long)(pair % top) * n_tokens + pair / top) * N;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -463,7 +469,8 @@ __global__ __launch_bounds__(256) void experts_gate_up_tiled_kernel(const T* __r
                                                                     const T* __restrict__ w_up, int F, int K, int top,
                                                                     const int* __restrict__ order,
                                                                     const int* __restrict__ tiles, float limit, float alpha,
-                                                                    float shift, T* __restrict__ act, long ldy) {
+                                                                    float shift, const float* __restrict__ in_weight,
+                                                                    T* __restrict__ act, long ldy) {
   __shared__ __attribute__((aligned(16))) char lds[2 * 3 * 64 * kLdsRow];
   const int e = tiles[4 * blockIdx.x];
   if (e < 0) return;
@@ -487,14 +494,15 @@ __global__ __launch_bounds__(256) void experts_gate_up_tiled_kernel(const T* __r
     const int r = wr * 32 + rt * 16 + l16;
     if (r >= rows) continue;
     T* dst = act + (long)(first + r) * ldy;
+    const float wt = in_weight ? in_weight[order[first + r]] : 1.0f;
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = col0 + wc * 32 + ct * 16 + 4 * quad + i;
         if (c < F) {
-          const float g = fminf(product.acc[0][rt][ct][i], limit);
-          const float u = fminf(fmaxf(product.acc[1][rt][ct][i], -limit), limit);
+          const float g = fminf(product.acc[0][rt][ct][i] * wt, limit);
+          const float u = fminf(fmaxf(product.acc[1][rt][ct][i] * wt, -limit), limit);
           dst[c] = from_f32<T>((g * sigmoid_e(alpha * g)) * (u + shift));
         }
       }
@@ -529,7 +537,7 @@ __global__ __launch_bounds__(256) void experts_down_tiled_kernel(const T* __rest
     const int r = wr * 32 + rt * 16 + l16;
     if (r >= rows) continue;
     const int pair = order[first + r];
-    const float share = weight[pair];
+    const float share = weight ? weight[pair] : 1.0f;
     float* dst = P + ((long)(pair % top) * n_tokens + pair / top) * N;
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct)
@@ -559,7 +567,8 @@ extern "C" int ls_experts_tile_capacity(int n_tokens, int E, int top, int rows_a
 // tiles [cap][4]; counts: scratch of E ints.  rows_a_tile 16, 32 or 64.
 extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int n_tokens, int E, int top,
                                 int rows_a_tile, int* expert, float* weight, int* order, int* tiles, int cap,
-                                int* counts, void* stream) {
+                                int* counts, int scoring, void* stream) {
+  LS_REQUIRE(scoring == 0 || scoring == 1, "experts_route: scoring %d (0: softmax over the chosen, 1: sigmoid)", scoring);
   LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && top <= E && top <= kMaxTop && ldz >= E,
              "experts_route: %d tokens, %d experts, %d chosen (at most %d)", n_tokens, E, top, kMaxTop);
   LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_route: tiles of %d rows", rows_a_tile);
@@ -570,10 +579,10 @@ extern "C" int ls_experts_route(const float* z, long ldz, const float* bias, int
   const int P = n_tokens * top;
   if (P <= kSmallPairs && E <= kSmallExperts) {
     hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(1024), 0, s, z, ldz, bias, n_tokens, E, top, rows_a_tile,
-                       expert, weight, order, tiles, cap, (const int*)nullptr, (const int*)nullptr);
+                       expert, weight, order, tiles, cap, (const int*)nullptr, (const int*)nullptr, scoring);
   } else {
     hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, s, z, ldz, bias, n_tokens, E, top,
-                       expert, weight);
+                       expert, weight, scoring);
     hipLaunchKernelGGL(route_count_kernel, dim3(E), dim3(64), 0, s, expert, P, counts);
     hipLaunchKernelGGL(route_place_kernel, dim3(E), dim3(64), 0, s, expert, counts, P, E, rows_a_tile, order, tiles, cap);
   }
@@ -592,7 +601,7 @@ extern "C" int ls_experts_route_table(const int* token_ids, const int* table, in
   const int P = n_tokens * top;
   if (P <= kSmallPairs && E <= kSmallExperts) {
     hipLaunchKernelGGL(route_small_kernel, dim3(1), dim3(1024), 0, s, (const float*)nullptr, 0L, (const float*)nullptr,
-                       n_tokens, E, top, rows_a_tile, expert, weight, order, tiles, cap, token_ids, table);
+                       n_tokens, E, top, rows_a_tile, expert, weight, order, tiles, cap, token_ids, table, 0);
   } else {
     hipLaunchKernelGGL(route_table_kernel, dim3((P + 255) / 256), dim3(256), 0, s, token_ids, table, n_tokens, top, expert,
                        weight);
@@ -607,7 +616,11 @@ extern "C" int ls_experts_route_table(const int* token_ids, const int* table, in
 extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* w_gate, const void* w_up,
                                 const void* w_down, int n_tokens, int E, int top, int K, int F, int N,
                                 int rows_a_tile, const int* order, const int* tiles, int cap, const float* weight,
-                                float limit, float alpha, float shift, void* act, long ldy, float* P, void* stream) {
+                                float limit, float alpha, float shift, void* act, long ldy, float* P, int weigh_input,
+                                void* stream) {
+  // weigh_input: the routing weight multiplies the expert's input instead of its output
+  const float* in_weight = weigh_input ? weight : nullptr;
+  const float* out_weight = weigh_input ? nullptr : weight;
   LS_REQUIRE(n_tokens > 0 && E > 0 && top > 0 && K > 0 && F > 0 && N > 0 && ldx >= K && ldy >= F, "experts_apply: bad sizes");
   LS_REQUIRE(rows_a_tile == 16 || rows_a_tile == 32 || rows_a_tile == 64, "experts_apply: tiles of %d rows", rows_a_tile);
   LS_REQUIRE(x && w_gate && w_up && w_down && order && tiles && weight && act && P && cap > 0, "experts_apply: null operand");
@@ -625,18 +638,20 @@ extern "C" int ls_experts_apply(int dtype, const void* x, long ldx, const void* 
 #define LS_EXPERTS(T_, RT_, KS_)                                                                                      \
   do {                                                                                                                \
     hipLaunchKernelGGL((experts_gate_up_kernel<T_, RT_, KS_>), grid_up, dim3(256), 0, s, (const T_*)x, ldx,           \
-                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, (T_*)act, ldy);     \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, in_weight,   \
+                       (T_*)act, ldy);                                                                                \
     hipLaunchKernelGGL((experts_down_kernel<T_, RT_, KS_>), grid_down, dim3(256), 0, s, (const T_*)act, ldy,          \
-                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
+                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, out_weight, P);                          \
   } while (0)
   // tiles of 64 rows go through LDS where every row of every operand starts on a 16-byte boundary
   const bool staged = rows_a_tile == 64 && K % vec == 0 && F % vec == 0 && ldx % vec == 0 && ldy % vec == 0;
 #define LS_EXPERTS_STAGED(T_)                                                                                         \
   do {                                                                                                                \
     hipLaunchKernelGGL(experts_gate_up_tiled_kernel<T_>, grid_up, dim3(256), 0, s, (const T_*)x, ldx,                 \
-                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, (T_*)act, ldy);     \
+                       (const T_*)w_gate, (const T_*)w_up, F, K, top, order, tiles, limit, alpha, shift, in_weight,   \
+                       (T_*)act, ldy);                                                                                \
     hipLaunchKernelGGL(experts_down_tiled_kernel<T_>, grid_down, dim3(256), 0, s, (const T_*)act, ldy,                \
-                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, weight, P);                              \
+                       (const T_*)w_down, N, F, top, n_tokens, order, tiles, out_weight, P);                          \
   } while (0)
 #define LS_EXPERTS_BY_ROWS(T_)                 \
   switch (rows_a_tile) {                       \

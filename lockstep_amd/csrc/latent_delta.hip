@@ -314,13 +314,24 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(
     const float* __restrict__ taps, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float unit_eps,
     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
     const float* __restrict__ state, long state_stride, long conv_at, float* __restrict__ qk, float* __restrict__ vv,
-    float* __restrict__ gates) {
-  const int units = 2 * G + H + 1;
+    float* __restrict__ gates, const float* __restrict__ chan, long ldc, float* __restrict__ decays) {
+  // (with a decay a key channel, chan [T][ldc] holds its H * D logits and dt_bias has as many entries: a unit a head
+  // then forms the head's beta and its row of decays, decays [T][H][dp], ones beyond D)
+  const int units = 2 * G + H + (chan ? H : 1);
   const long id = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (id >= (long)n_tokens * units) return;
   const int t = (int)(id / units), unit = (int)(id % units), lane = threadIdx.x & 63;
   const float* row = raw + (long)t * ld;
   const int C = 2 * G * D + H * DV;
+  if (chan && unit >= 2 * G + H) {
+    const int h = unit - (2 * G + H);
+    if (lane < 2) gates[((long)t * H + h) * 2 + lane] = lane == 0 ? sigmoid_f(row[C + h]) : 1.0f;
+    const float rate = expf(a_log[h]);
+    for (int r = lane; r < dp; r += 64)
+      decays[((long)t * H + h) * dp + r] =
+          r < D ? expf(-rate * softplus_f(chan[(long)t * ldc + h * D + r] + dt_bias[h * D + r])) : 1.0f;
+    return;
+  }
   if (unit == units - 1) {
     for (int h = lane; h < H; h += 64) {
       gates[((long)t * H + h) * 2] = sigmoid_f(row[C + h]);
@@ -381,10 +392,12 @@ __device__ __forceinline__ float lanes_sum(float v) {
   return v;
 }
 
-// R rows a lane, L lanes a column (R * L rows, the head size rounded up), 64 / L columns a wave.
-template <int R, int L>
+// R rows a lane, L lanes a column (R * L rows, the head size rounded up), 64 / L columns a wave.  CH: the decay is a
+// number a row of the state (decays [T][H][dp]) instead of one a head: S[r] <- g[r] S[r] first, then the rule as stated.
+template <int R, int L, bool CH>
 __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict__ qk, const float* __restrict__ vv,
-                                                        const float* __restrict__ gates, int G, int H, int D, int DV,
+                                                        const float* __restrict__ gates, const float* __restrict__ decays,
+                                                        int G, int H, int D, int DV,
                                                         const SeqMeta* __restrict__ seqs, float* __restrict__ state,
                                                         long state_stride, float* __restrict__ out, long ldo) {
   constexpr int dp = L * R, COLS = 64 / L;
@@ -401,7 +414,7 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
 #pragma unroll
   for (int r = 0; r < R; ++r) S[r] = (row0 + r < D && col_ok) ? mine[(long)(row0 + r) * DV + col] : 0.f;
   struct Operands {
-    f32x4 q[R / 4], k[R / 4];
+    f32x4 q[R / 4], k[R / 4], g[CH ? R / 4 : 1];
     float v, gate;   // gate: beta in the even lanes, the decay in the odd ones
   };
   // Pointers to the operands of the token that is requested next; they move on by a token after every request and
@@ -413,6 +426,7 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
   const float* k_at = q_at + (long)G * dp;
   const float* v_at = vv + (long)m.q_off * H * DV + head * DV + (col_ok ? col : 0);
   const float* g_at = gates + ((long)m.q_off * H + head) * 2 + (lane & 1);
+  const float* d_at = CH ? decays + ((long)m.q_off * H + head) * dp + row0 : nullptr;
   int left = m.q_len - 1;   // tokens behind the one the pointers stand on
   auto fetch = [&]() LS_INLINED {
     Operands x;
@@ -420,6 +434,7 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
     for (int j = 0; j < R / 4; ++j) {
       x.q[j] = *reinterpret_cast<const f32x4*>(q_at + 4 * j);
       x.k[j] = *reinterpret_cast<const f32x4*>(k_at + 4 * j);
+      if constexpr (CH) x.g[j] = *reinterpret_cast<const f32x4*>(d_at + 4 * j);
     }
     x.v = *v_at;
     x.gate = *g_at;
@@ -429,10 +444,11 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
     k_at += step * 2 * G * dp;
     v_at += step * H * DV;
     g_at += step * H * 2;
+    if constexpr (CH) d_at += step * H * dp;
     return x;
   };
   // the operands of the token DEPTH tokens on are requested before a token is worked on (a ring of registers)
-  constexpr int DEPTH = R <= 8 ? 8 : 4;
+  constexpr int DEPTH = (R <= 8 && !CH) ? 8 : 4;
   Operands ring[DEPTH];
 #pragma unroll
   for (int j = 0; j < DEPTH; ++j) ring[j] = fetch();
@@ -447,14 +463,18 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(const float* __restrict_
       const float decay = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(now.gate), 0x55, 0xF, 0xF, true));  // lane 1
       // a lane's rows in four interleaved chains (rows r, r + 4, ... of each), added as (0 + 1) + (2 + 3)
       float ks4[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (CH) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) S[r] = S[r] * now.g[r >> 2][r & 3];
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) ks4[r & 3] = fmaf(S[r], now.k[r >> 2][r & 3], ks4[r & 3]);
-      const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * decay;
+      const float ks = lanes_sum<L>((ks4[0] + ks4[1]) + (ks4[2] + ks4[3])) * (CH ? 1.0f : decay);
       const float u = beta * (now.v - ks);
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        S[r] = fmaf(now.k[r >> 2][r & 3], u, decay * S[r]);
+        S[r] = fmaf(now.k[r >> 2][r & 3], u, CH ? S[r] : decay * S[r]);
         o4[r & 3] = fmaf(S[r], now.q[r >> 2][r & 3], o4[r & 3]);
       }
       const float o = lanes_sum<L>((o4[0] + o4[1]) + (o4[2] + o4[3]));
@@ -612,16 +632,24 @@ extern "C" int ls_delta_padded_dim(int D) {
 extern "C" long ls_delta_scratch_floats(int n_tokens, int G, int H, int D, int DV) {
   return (long)n_tokens * (2L * G * ls_delta_padded_dim(D) + (long)H * DV + 2L * H);
 }
+// ... and with a decay a key channel (chan given): the decays as well.
+extern "C" long ls_delta_scratch_floats_channel(int n_tokens, int G, int H, int D, int DV) {
+  return ls_delta_scratch_floats(n_tokens, G, H, D, DV) + (long)n_tokens * H * ls_delta_padded_dim(D);
+}
 
 extern "C" int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int H, int D, int DV, int M,
                              const float* taps, const float* a_log, const float* dt_bias, float unit_eps,
                              const int* tok_seq, const int* tok_pos, const void* seqs, int n_seqs, float* state,
-                             long state_stride, float* scratch, float* out, long ldo, void* stream) {
+                             long state_stride, float* scratch, float* out, long ldo, const float* chan, long ldc,
+                             void* stream) {
+  // chan [T][ldc] (or null): the logits of a decay a head and key channel, H * D a token; dt_bias then has H * D
+  // entries, raw needs no `a` columns, and the scratch is that of ls_delta_scratch_floats_channel.
+  LS_REQUIRE(!chan || ldc >= (long)H * D, "delta_rule: the channel decays' rows are too short");
   LS_REQUIRE(n_tokens > 0 && n_seqs > 0 && G > 0 && H > 0 && H % G == 0 && D > 0 && D <= 256 && DV > 0 && M >= 1,
              "delta_rule: bad sizes (%d key heads, %d heads, keys of %d, values of %d, %d taps)", G, H, D, DV, M);
   const long C = 2L * G * D + (long)H * DV;
   const long conv_at = (long)H * D * DV;
-  LS_REQUIRE(ld >= C + 2L * H && state_stride >= conv_at + (long)(M - 1) * C && ldo >= (long)H * DV,
+  LS_REQUIRE(ld >= C + (chan ? 1L : 2L) * H && state_stride >= conv_at + (long)(M - 1) * C && ldo >= (long)H * DV,
              "delta_rule: rows or state are too short");
   LS_REQUIRE(raw && taps && a_log && dt_bias && tok_seq && tok_pos && seqs && state && scratch && out,
              "delta_rule: null operand");
@@ -631,13 +659,20 @@ extern "C" int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int
   float* qk = scratch;
   float* vv = qk + (long)n_tokens * 2 * G * dp;
   float* gates = vv + (long)n_tokens * H * DV;
-  const long units = (long)n_tokens * (2 * G + H + 1);
+  float* decays = chan ? gates + (long)n_tokens * H * 2 : nullptr;
+  const long units = (long)n_tokens * (2 * G + H + (chan ? H : 1));
   hipLaunchKernelGGL(delta_prep_kernel, dim3((unsigned)((units + 3) / 4)), dim3(256), 0, s, raw, ld, n_tokens, G, H, D, DV,
                      dp, M, taps, a_log, dt_bias, unit_eps, tok_seq, tok_pos, (const SeqMeta*)seqs, state, state_stride,
-                     conv_at, qk, vv, gates);
+                     conv_at, qk, vv, gates, chan, ldc, decays);
 #define LS_DELTA(R_, L_)                                                                                              \
-  hipLaunchKernelGGL((delta_rule_kernel<R_, L_>), dim3(n_seqs * H, (DV * L_ + 63) / 64), dim3(64), 0, s, qk, vv, gates, G, H, \
-                     D, DV, (const SeqMeta*)seqs, state, state_stride, out, ldo)
+  do {                                                                                                                \
+    if (chan)                                                                                                         \
+      hipLaunchKernelGGL((delta_rule_kernel<R_, L_, true>), dim3(n_seqs * H, (DV * L_ + 63) / 64), dim3(64), 0, s, qk, vv, \
+                         gates, decays, G, H, D, DV, (const SeqMeta*)seqs, state, state_stride, out, ldo);            \
+    else                                                                                                              \
+      hipLaunchKernelGGL((delta_rule_kernel<R_, L_, false>), dim3(n_seqs * H, (DV * L_ + 63) / 64), dim3(64), 0, s, qk, vv, \
+                         gates, decays, G, H, D, DV, (const SeqMeta*)seqs, state, state_stride, out, ldo);            \
+  } while (0)
   switch (dp) {
     case 16: LS_DELTA(4, 4); break;
     case 32: LS_DELTA(8, 4); break;

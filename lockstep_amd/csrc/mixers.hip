@@ -161,7 +161,8 @@ __global__ __launch_bounds__(256) void talk_qkv_kernel(
 //   v = k as projected, with its bias, before any norm (keys_are_values; DV == D);
 //   q and k each divided by the root mean square over ALL their heads at once (the whole projection is one
 //   vector: x / sqrt(mean(x^2) + eps)), times a weight an element (q_norm [H*D], k_norm [G*D]; null: no norm);
-//   or, with per_head, every head of q and of k divided by its own root mean square over D (no weights);
+//   or, with per_head, every head of q and of k divided by its own root mean square over D (per_head 1: no weights;
+//   per_head 2: times q_norm [D] / k_norm [D], one weight vector that all heads share);
 //   q and k rotated on their first `rot` dimensions at the token's position, pairs (i, i + rot/2) or, with
 //   `neighbours`, (2i, 2i + 1), angle tables [positions][rot/2];
 //   q -> q_out [T][H*Dp] (T);  k -> key pages [page][G][slot][Dp], Dp >= D with zeros beyond D (a kernel that loads
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     }
     __syncthreads();
   }
-  if (q_norm) {
+  if (q_norm && !per_head) {
     float part = 0.f;
     for (int e = threadIdx.x; e < nq; e += 256) {
       const float x = row[e] + (bias ? bias[e] : 0.f);
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
     }
     rq = 1.0f / sqrtf(block_sum256(part, scratch) / (float)nq + eps);
   }
-  if (k_norm) {
+  if (k_norm && !per_head) {
     float part = 0.f;
     for (int e = threadIdx.x; e < nk; e += 256) {
       const float x = row[nq + e] + (bias ? bias[nq + e] : 0.f);
@@ -240,18 +241,21 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(
   // element e of q | k as the attention reads it: bias, norm, rotation
   auto finished = [&](int e) LS_INLINED {
     const bool is_q = e < nq;
-    const float* w = is_q ? q_norm : k_norm;
+    const float* w = per_head ? nullptr : (is_q ? q_norm : k_norm);
+    const float* hw = per_head == 2 ? (is_q ? q_norm : k_norm) : nullptr;   // a head's weights, shared by the heads
     const int at = is_q ? e : e - nq;      // index into the norm weight
     const float r = is_q ? rq : rk;
     float own = row[e] + (bias ? bias[e] : 0.f);
+    const int i = e % D;
     if (w) own = own * r * w[at];
     if (per_head) own = own * head_scale[e / D];
-    const int i = e % D;
+    if (hw) own = own * hw[i];
     if (i < rot) {
       const int pe = neighbours ? (e ^ 1) : (i < half ? e + half : e - half);
       float other = row[pe] + (bias ? bias[pe] : 0.f);
       if (w) other = other * r * w[is_q ? pe : pe - nq];
       if (per_head) other = other * head_scale[e / D];
+      if (hw) other = other * hw[pe % D];
       const int pair = neighbours ? (i >> 1) : (i < half ? i : i - half);
       const bool lower = neighbours ? (i & 1) == 0 : i < half;
       own = lower ? own * cos_row[pair] - other * sin_row[pair] : own * cos_row[pair] + other * sin_row[pair];
@@ -500,14 +504,14 @@ __global__ __launch_bounds__(1024) void linrec_kernel(const float* __restrict__ 
 
 // ---------------------------------------------------------------------------
 // Per (token, head): x [DV] float divided by its root mean square (eps inside the root), times
-// weight[c] if given, times silu(gate[t][head * DV + c]) if given; stored as T.  One wave a
+// weight[c] if given, times silu (gate_act 0) or sigmoid (gate_act 1) of gate[t][head * DV + c] if given; stored as T.  One wave a
 // head: lane i adds the squares of the elements i, i + 64, ... ascending, then a butterfly.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ x, long ldx, int n_tokens,
                                                              int H, int DV, const float* __restrict__ weight,
-                                                             const float* __restrict__ gate, long ldg, float eps,
-                                                             T* __restrict__ out, long ldo) {
+                                                             const float* __restrict__ gate, long ldg, int gate_act,
+                                                             float eps, T* __restrict__ out, long ldo) {
   const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (unit >= (long)n_tokens * H) return;
   const int t = (int)(unit / H), head = (int)(unit % H), lane = threadIdx.x & 63;
@@ -519,9 +523,71 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   for (int c = lane; c < DV; c += 64) {
     float v = src[c] * scale;
     if (weight) v = v * weight[c];
-    if (gate) v = v * siluf_(gate[(long)t * ldg + head * DV + c]);
+    if (gate) {
+      const float z = gate[(long)t * ldg + head * DV + c];
+      v = v * (gate_act == 1 ? sigmoidf_(z) : siluf_(z));
+    }
     out[(long)t * ldo + head * DV + c] = from_f32<T>(v);
   }
+}
+
+// ---------------------------------------------------------------------------
+// Embedding with a second table indexed by a hash of the token and the token before it:
+//   out[t] = E[token[t]] * scale + B[(token[t-1] * mul_prev + token[t] * mul_cur) mod buckets],   row `buckets` of B
+// for a request's first token.  The token before a portion's first one is the request's state (one int a slot):
+// the workgroup of that row reads it and then leaves the portion's last token there for the next step (no other
+// workgroup touches the slot).  One workgroup a token.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void embed_pair_kernel(const int* __restrict__ tokens, const int* __restrict__ tok_seq,
+                                                         const int* __restrict__ tok_pos, const SeqMeta* __restrict__ seqs,
+                                                         const T* __restrict__ table, const T* __restrict__ pairs,
+                                                         int buckets, long mul_prev, long mul_cur, int* __restrict__ state,
+                                                         long state_stride, float* __restrict__ out, int width,
+                                                         long ld_out, float scale) {
+  const int t = blockIdx.x;
+  const SeqMeta m = seqs[tok_seq[t]];
+  const bool first_row = t == m.q_off;
+  const int token = tokens[t];
+  int* kept = state + (long)m.table_row * state_stride;
+  const int before = first_row ? kept[0] : tokens[t - 1];
+  long row = buckets;
+  if (tok_pos[t] > 0) {
+    row = ((long)before * mul_prev + (long)token * mul_cur) % buckets;
+    if (row < 0) row += buckets;     // (a slot that was never written must not lead outside the table)
+  }
+  const T* e_row = table + (long)token * width;
+  const T* p_row = pairs + row * width;
+  float* dst = out + (long)t * ld_out;
+  for (int c = threadIdx.x; c < width; c += 256) dst[c] = to_f32(e_row[c]) * scale + to_f32(p_row[c]);
+  if (first_row) {
+    __syncthreads();                 // every thread has read the slot
+    if (threadIdx.x == 0) kept[0] = tokens[m.q_off + m.q_len - 1];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Token shift: a sublayer's input h[t] is replaced by h[t] + (h[t-1] - h[t]) * mu, element by element, with h[t-1]
+// the unshifted input of the token before (zeros for a request's first token).  n [T][ldn] float holds the unshifted
+// inputs of the step; the input of the token before a portion's first one is the request's state (width floats a
+// slot), which the threads of that row read and then overwrite with the portion's last input.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_kernel(const float* __restrict__ n, long ldn, const float* __restrict__ mu,
+                                                          const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                          const SeqMeta* __restrict__ seqs, float* __restrict__ state,
+                                                          long state_stride, T* __restrict__ out, long ldo, int width) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= width) return;
+  const SeqMeta m = seqs[tok_seq[t]];
+  const bool first_row = t == m.q_off;
+  float* kept = state + (long)m.table_row * state_stride;
+  const float own = n[(long)t * ldn + c];
+  float before = first_row ? kept[c] : n[(long)(t - 1) * ldn + c];
+  if (tok_pos[t] == 0) before = 0.f;
+  out[(long)t * ldo + c] = from_f32<T>(own + (before - own) * mu[c]);
+  if (first_row) kept[c] = n[(long)(m.q_off + m.q_len - 1) * ldn + c];
 }
 
 }  // namespace ls
@@ -551,6 +617,45 @@ extern "C" int ls_dyt(int dtype, float* h, const float* P, int slices, int p_row
   else
     return fail("dyt: unknown dtype %d", dtype);
   return check_launch("dyt");
+}
+
+extern "C" int ls_embed_pair(int dtype, const int* tokens, const int* tok_seq, const int* tok_pos, const void* seqs,
+                             const void* table, int vocab, const void* pairs, int buckets, long mul_prev, long mul_cur,
+                             int* state, long state_stride, float* out, int n_tokens, int width, long ld_out, float scale,
+                             void* stream) {
+  LS_REQUIRE(n_tokens > 0 && vocab > 0 && width > 0 && buckets > 0 && ld_out >= width && state_stride >= 1,
+             "embed_pair: bad sizes");
+  LS_REQUIRE(tokens && tok_seq && tok_pos && seqs && table && pairs && state && out, "embed_pair: null operand");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    hipLaunchKernelGGL(embed_pair_kernel<float>, dim3(n_tokens), dim3(256), 0, s, tokens, tok_seq, tok_pos,
+                       (const SeqMeta*)seqs, (const float*)table, (const float*)pairs, buckets, mul_prev, mul_cur, state,
+                       state_stride, out, width, ld_out, scale);
+  else if (dtype == kBF16)
+    hipLaunchKernelGGL(embed_pair_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, s, tokens, tok_seq, tok_pos,
+                       (const SeqMeta*)seqs, (const bf16_t*)table, (const bf16_t*)pairs, buckets, mul_prev, mul_cur, state,
+                       state_stride, out, width, ld_out, scale);
+  else
+    return fail("embed_pair: unknown dtype %d", dtype);
+  return check_launch("embed_pair");
+}
+
+extern "C" int ls_token_shift(int out_dtype, const float* n, long ldn, const float* mu, const int* tok_seq,
+                              const int* tok_pos, const void* seqs, float* state, long state_stride, void* out, long ldo,
+                              int n_tokens, int width, void* stream) {
+  LS_REQUIRE(n_tokens > 0 && width > 0 && ldn >= width && ldo >= width && state_stride >= width, "token_shift: bad sizes");
+  LS_REQUIRE(n && mu && tok_seq && tok_pos && seqs && state && out, "token_shift: null operand");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)n_tokens, (unsigned)((width + 255) / 256));
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL(token_shift_kernel<float>, grid, dim3(256), 0, s, n, ldn, mu, tok_seq, tok_pos, (const SeqMeta*)seqs,
+                       state, state_stride, (float*)out, ldo, width);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL(token_shift_kernel<bf16_t>, grid, dim3(256), 0, s, n, ldn, mu, tok_seq, tok_pos,
+                       (const SeqMeta*)seqs, state, state_stride, (bf16_t*)out, ldo, width);
+  else
+    return fail("token_shift: unknown dtype %d", out_dtype);
+  return check_launch("token_shift");
 }
 
 extern "C" int ls_glu_clamped(int out_dtype, const float* x, long ldx, void* out, long ldo, int rows, int width,
@@ -627,8 +732,9 @@ extern "C" int ls_qkv_post(int dtype, const float* raw, long ld, int n_tokens, i
              "qkv_post: position %d is beyond the rotation tables (%d)", max_pos, table_positions);
   LS_REQUIRE(max_pos / page_size < table_stride, "qkv_post: position %d is beyond the block table", max_pos);
   LS_REQUIRE((q_norm == nullptr) == (k_norm == nullptr) && (!q_norm || eps > 0.f), "qkv_post: bad norm");
-  LS_REQUIRE(!per_head || (!q_norm && eps > 0.f && H + G <= kMaxNormedHeads),
-             "qkv_post: a norm a head has no weights and takes up to %d heads", kMaxNormedHeads);
+  LS_REQUIRE(!per_head || (((per_head == 1 && !q_norm) || (per_head == 2 && q_norm)) && eps > 0.f && H + G <= kMaxNormedHeads),
+             "qkv_post: a norm a head has no weights (1) or one weight vector for all heads (2), and takes up to %d heads",
+             kMaxNormedHeads);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   // Without a norm every element stands alone: a thread an element.  With one, every workgroup of a token forms the
   // row's sums itself, so a step of many tokens gives each token one workgroup, and a few tokens are spread out.
@@ -696,19 +802,19 @@ extern "C" int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_a
 }
 
 extern "C" int ls_head_norm_gate(int out_dtype, const float* x, long ldx, int n_tokens, int H, int DV,
-                                 const float* weight, const float* gate, long ldg, float eps, void* out, long ldo,
-                                 void* stream) {
+                                 const float* weight, const float* gate, long ldg, int gate_act, float eps, void* out,
+                                 long ldo, void* stream) {
   LS_REQUIRE(n_tokens > 0 && H > 0 && DV > 0 && x && out && ldx >= (long)H * DV && ldo >= (long)H * DV &&
-                 (!gate || ldg >= (long)H * DV),
+                 (!gate || ldg >= (long)H * DV) && (gate_act == 0 || gate_act == 1),
              "head_norm_gate: bad sizes");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   dim3 grid((unsigned)(((long)n_tokens * H + 3) / 4));
   if (out_dtype == kF32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, dim3(256), 0, s, x, ldx, n_tokens, H, DV, weight, gate, ldg,
-                       eps, (float*)out, ldo);
+                       gate_act, eps, (float*)out, ldo);
   else if (out_dtype == kBF16)
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, dim3(256), 0, s, x, ldx, n_tokens, H, DV, weight, gate,
-                       ldg, eps, (bf16_t*)out, ldo);
+                       ldg, gate_act, eps, (bf16_t*)out, ldo);
   else
     return fail("head_norm_gate: unknown dtype %d", out_dtype);
   return check_launch("head_norm_gate");

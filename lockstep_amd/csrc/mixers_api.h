@@ -52,9 +52,22 @@ int ls_linrec(int mode, const float* raw, long ld, int q_at, int ab_at, int v_at
               int table_positions, int max_pos, const int* tok_pos, const void* seqs, int n_seqs, float* state,
               float* gates, float* out, long ldo, void* stream);
 
-// Per (token, head): x [DV] / sqrt(mean(x^2) + eps), times weight [DV] and silu(gate) where given.
+// Per (token, head): x [DV] / sqrt(mean(x^2) + eps), times weight [DV] and silu(gate) (gate_act 0) or sigmoid(gate)
+// (gate_act 1) where given.
 int ls_head_norm_gate(int out_dtype, const float* x, long ldx, int n_tokens, int H, int DV, const float* weight,
-                      const float* gate, long ldg, float eps, void* out, long ldo, void* stream);
+                      const float* gate, long ldg, int gate_act, float eps, void* out, long ldo, void* stream);
+
+// out [T][ld_out] float = table[token] * scale + pairs[(token before * mul_prev + token * mul_cur) mod buckets]; row
+// `buckets` of pairs for a request's first token.  state: one int a slot, the last token of the request so far.
+int ls_embed_pair(int dtype, const int* tokens, const int* tok_seq, const int* tok_pos, const void* seqs, const void* table,
+                  int vocab, const void* pairs, int buckets, long mul_prev, long mul_cur, int* state, long state_stride,
+                  float* out, int n_tokens, int width, long ld_out, float scale, void* stream);
+
+// out [T][ldo] = n[t] + (n[t-1] - n[t]) * mu, n [T][ldn] float; the row before a portion's first one is the request's
+// state (width floats a slot; zeros at a request's first token), which is left as the portion's last row.
+int ls_token_shift(int out_dtype, const float* n, long ldn, const float* mu, const int* tok_seq, const int* tok_pos,
+                   const void* seqs, float* state, long state_stride, void* out, long ldo, int n_tokens, int width,
+                   void* stream);
 
 // A residual stream of n copies X [rows][n][width] float.  Write (P given): y = P[0][row] + P[1][row] + ..., then
 // X'_t = sum_s mix[s][t] X_s + gain[t] y for all copies at once.  Read (out given): u = sum_t take[t] X'_t (take null:
@@ -90,10 +103,13 @@ int ls_heads_product(int dtype, const void* x, long ldx, int x_stride, const voi
 int ls_delta_max_dim();
 int ls_delta_padded_dim(int D);
 long ls_delta_scratch_floats(int n_tokens, int G, int H, int D, int DV);
+long ls_delta_scratch_floats_channel(int n_tokens, int G, int H, int D, int DV);
+// chan [T][ldc] float or null: logits of a decay a head and key channel (H * D a token; dt_bias [H * D]; raw then ends
+// with b; scratch of ls_delta_scratch_floats_channel floats): g = exp(-exp(A_log_h) softplus(chan + dt_bias)).
 int ls_delta_rule(const float* raw, long ld, int n_tokens, int G, int H, int D, int DV, int M, const float* taps,
                   const float* a_log, const float* dt_bias, float unit_eps, const int* tok_seq, const int* tok_pos,
                   const void* seqs, int n_seqs, float* state, long state_stride, float* scratch, float* out, long ldo,
-                  void* stream);
+                  const float* chan, long ldc, void* stream);
 
 int ls_listed_index(const char* name);
 int ls_call_listed(int index, const long long* words, int n);

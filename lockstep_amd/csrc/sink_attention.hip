@@ -2,7 +2,9 @@
 // sees and of what is added to its scores:
 //
 //   s_h[i, j]    = (q_h[i] . k_kv(h)[j]) * scale + bias_h[min(i - j, n_dist - 1)]   (bias optional)
-//   visible(i,j) = lo(i) <= j <= i,   lo(i) = max(window ? i - window + 1 : 0, chunk ? floor(i / chunk) chunk : 0)
+//   visible(i,j) = lo(i) <= j <= i,   lo(i) = max(window ? i - window + 1 : 0, chunk ? floor(i / chunk) chunk : 0),
+//                  or j < keep_first (the first tokens stay visible when a window has passed them; their tiles are
+//                  walked before the window's)
 //   p_h[i, j]    = exp(s_h[i, j]) / (exp(sink_h) + sum over visible j' of exp(s_h[i, j']))  (without a sink: no term)
 //   o_h[i]       = gate_h[i] * sum_j p_h[i, j] v_kv(h)[j],   gate = sigmoid(g_h[i]) elementwise (optional)
 //
@@ -72,7 +74,7 @@ template <typename T, int RT, bool DEC>
 __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
     const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ items,
-    int H, int G, float scale, int window, int chunk, const float* __restrict__ sink,
+    int H, int G, float scale, int window, int chunk, int keep_first, const float* __restrict__ sink,
     const float* __restrict__ dist_bias, int n_dist, const float* __restrict__ gate, long ldg, T* __restrict__ out,
     long ldo, float* __restrict__ part, int part_rows) {
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
@@ -123,7 +125,9 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   const int lo_last = first_seen(p_last, window, chunk);   // (no row of the block begins to see later than this)
   const int lo_tile = first_seen(p_first, window, chunk) / kTileKeys;
   const int hi_tile = p_last / kTileKeys;
-  const int n_tiles = hi_tile - lo_tile + 1;
+  const int kept_tiles = min((keep_first + kTileKeys - 1) / kTileKeys, lo_tile);   // tiles of kept first tokens below the window's
+  const int n_tiles = kept_tiles + hi_tile - lo_tile + 1;
+  auto tile_at = [&](int step) LS_INLINED { return step < kept_tiles ? step : lo_tile + (step - kept_tiles); };
   const int per_run = (n_tiles + n_runs - 1) / n_runs;
   const int step_end = min(n_tiles, (run + 1) * per_run);
 
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
     v4_t vv[2][kAheadV ? VB : 1];
   };
   auto request = [&](int step, Ahead& t) LS_INLINED {
-    const int key0 = (lo_tile + step) * kTileKeys;
+    const int key0 = tile_at(step) * kTileKeys;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int key = key0 + 16 * half + l16;
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
   Ahead now;
   if (run * per_run < step_end) request(run * per_run, now);
   for (int step = run * per_run; step < step_end; ++step) {
-    const int key0 = (lo_tile + step) * kTileKeys;
+    const int key0 = tile_at(step) * kTileKeys;
     bool v_ok[2][4];
     long v_at[2];
     v4_t vv[2][kAheadV ? VB : 1];
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = key0 + 16 * half + 4 * quad + i;
-            see[half][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
+            see[half][i] = kWhole || (row_ok[r] && key <= my_pos[r] && (key >= my_lo[r] || key < keep_first));
             float v = s[r][half][i] * scale;
             if constexpr (kBiased) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
             s[r][half][i] = v;
@@ -257,7 +261,7 @@ __global__ __launch_bounds__(64 * (DEC ? 1 : kMaxWaves)) void sink_attention_ker
       }
     };
     // (the mask and the bias are instances of the code, chosen by scalar branches once a tile)
-    const bool whole_tile = key0 + kTileKeys - 1 <= p_first && key0 >= lo_last;
+    const bool whole_tile = key0 + kTileKeys - 1 <= p_first && (key0 >= lo_last || key0 + kTileKeys <= keep_first);
     if (my_bias) {
       if (whole_tile) softmax_tile(std::true_type{}, std::true_type{});
       else softmax_tile(std::false_type{}, std::true_type{});
@@ -404,7 +408,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
     const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ items,
-    int H, int G, float scale, int window, int chunk, const float* __restrict__ sink,
+    int H, int G, float scale, int window, int chunk, int keep_first, const float* __restrict__ sink,
     const float* __restrict__ dist_bias, int n_dist, const float* __restrict__ gate, long ldg, T* __restrict__ out,
     long ldo, float* __restrict__ part, int part_rows) {
   typedef typename Atom<T>::vec_t vec_t;
@@ -475,7 +479,9 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
 
   const int lo_tile = first_seen(p_first, window, chunk) / TK;
   const int hi_tile = p_last / TK;
-  const int n_tiles = hi_tile - lo_tile + 1;
+  const int kept_tiles = min((keep_first + TK - 1) / TK, lo_tile);   // tiles of kept first tokens below the window's
+  const int n_tiles = kept_tiles + hi_tile - lo_tile + 1;
+  auto tile_at = [&](int step) LS_INLINED { return step < kept_tiles ? step : lo_tile + (step - kept_tiles); };
   const int per_run = (n_tiles + n_runs - 1) / n_runs;
   const int step_begin = run * per_run, step_end = min(n_tiles, (run + 1) * per_run);
 
@@ -484,13 +490,13 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
   // (pages of at least a tile's keys: one page a tile)
   const int tile_pages = max(1, TK >> page_shift);
   auto look_up = [&](int step) LS_INLINED {       // thread i: the page of the tile's i-th run of keys, -1 beyond the block
-    const int key0 = (lo_tile + step) * TK;
+    const int key0 = tile_at(step) * TK;
     const int key = max(key0, ((key0 >> page_shift) + (int)threadIdx.x) << page_shift);
     const bool in = (int)threadIdx.x < tile_pages && step < step_end && key <= p_last;
     return in ? my_table[key >> page_shift] : -1;
   };
   auto request = [&](int step) LS_INLINED {
-    const int key0 = (lo_tile + step) * TK;
+    const int key0 = tile_at(step) * TK;
     const int* pages = page_s[step & 1];
     const int first_page = key0 >> page_shift;
 #pragma unroll
@@ -542,7 +548,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
   }
   __syncthreads();
   for (int step = step_begin; step < step_end; ++step) {
-    const int key0 = (lo_tile + step) * TK;
+    const int key0 = tile_at(step) * TK;
     const int page_after = threadIdx.x < kTilePages ? look_up(step + 2) : -1;   // (on its way during the tile)
     if (step + 1 < step_end) request(step + 1);
     if (active && key0 <= wave_last) {
@@ -575,7 +581,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               const int key = key0 + 16 * ng + 4 * quad + i;
-              see[ng][i] = kWhole || (row_ok[r] && key <= my_pos[r] && key >= my_lo[r]);
+              see[ng][i] = kWhole || (row_ok[r] && key <= my_pos[r] && (key >= my_lo[r] || key < keep_first));
               float v = s[r][ng][i] * scale;
               if constexpr (kBiased) v = v + my_bias[min(max(my_pos[r] - key, 0), n_dist - 1)];
               s[r][ng][i] = v;
@@ -598,7 +604,7 @@ __global__ __launch_bounds__(256) void sink_attention_staged_kernel(
           moved = moved || shrink[r] != 1.0f;
         }
       };
-      const bool whole_tile = key0 + TK - 1 <= wave_first && key0 >= wave_lo_last;
+      const bool whole_tile = key0 + TK - 1 <= wave_first && (key0 >= wave_lo_last || key0 + TK <= keep_first);
       if (my_bias) {
         if (whole_tile) softmax_tile(std::true_type{}, std::true_type{});
         else softmax_tile(std::false_type{}, std::true_type{});
@@ -779,7 +785,7 @@ extern "C" int ls_sink_staged_rows(int H, int G) {
 extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void* k_pages, const void* v_pages,
                                  int page_size, const int* table, int table_stride, const void* seqs,
                                  const int* items, int n_items, int row_tiles, int H, int G, float scale, int window,
-                                 int chunk, const float* sink, const float* dist_bias, int n_dist, const float* gate,
+                                 int chunk, int keep_first, const float* sink, const float* dist_bias, int n_dist, const float* gate,
                                  long ldg, void* out, long ldo, const int* folds, int n_folds, float* part,
                                  int part_rows, void* stream) {
   LS_REQUIRE(row_tiles == 0 || row_tiles == 1 || row_tiles == 2 || row_tiles == 4 || row_tiles == 8,
@@ -796,6 +802,8 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
              "sink_attention: page size %d is not a power of two", page_size);
   LS_REQUIRE(window >= 0 && chunk >= 0 && (!dist_bias || n_dist > 0), "sink_attention: window %d, chunk %d, %d distances",
              window, chunk, n_dist);
+  LS_REQUIRE(keep_first >= 0 && (keep_first == 0 || (window > 0 && chunk == 0)),
+             "sink_attention: %d kept first tokens need a window (and no chunks)", keep_first);
   LS_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
                  reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
              "sink_attention: operands must be 16-byte aligned");
@@ -808,13 +816,13 @@ extern "C" int ls_sink_attention(int dtype, const void* q, long ldq, const void*
                      dim3(n_items, G, DEC_ ? (GS + 15) / 16 : (GS + kMaxWaves - 1) / kMaxWaves),                       \
                      dim3(DEC_ ? 64 : 64 * (GS < kMaxWaves ? GS : kMaxWaves)), 0, s, (const T_*)q, ldq,                \
                      (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride, (const SeqMeta*)seqs,     \
-                     items, H, G, scale, window, chunk, sink, dist_bias, n_dist, gate, ldg, (T_*)out, ldo, part,       \
-                     part_rows)
+                     items, H, G, scale, window, chunk, keep_first, sink, dist_bias, n_dist, gate, ldg, (T_*)out, ldo, \
+                     part, part_rows)
 #define LS_SINK_STAGED(T_)                                                                                             \
   hipLaunchKernelGGL(sink_attention_staged_kernel<T_>, dim3(n_items, G, (GS + 3) / 4), dim3(256), 0, s, (const T_*)q,  \
                      ldq, (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride,                      \
-                     (const SeqMeta*)seqs, items, H, G, scale, window, chunk, sink, dist_bias, n_dist, gate, ldg,      \
-                     (T_*)out, ldo, part, part_rows)
+                     (const SeqMeta*)seqs, items, H, G, scale, window, chunk, keep_first, sink, dist_bias, n_dist,     \
+                     gate, ldg, (T_*)out, ldo, part, part_rows)
 #define LS_SINK_BY_ROWS(T_)                       \
   switch (row_tiles) {                            \
     case 0: LS_SINK_LAUNCH(T_, 1, true); break;   \

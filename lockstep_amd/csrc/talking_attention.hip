@@ -25,6 +25,18 @@
 // times the keys of the early ones): a row block's tiles are dealt to several work items in
 // contiguous runs, each leaves (max, sum, unnormalised output) of its run for every row, and a
 // second kernel folds the runs in ascending order.
+//
+// A second way of talking mixes the heads' WEIGHTS, after each head's own softmax (MODE 1 and 2 of the kernel):
+//
+//   p_g[i, j]    = exp(raw_g[i, j]) / (exp(sink_g) + sum over visible j' of exp(raw_g[i, j']))     (the sink is optional)
+//   w_h[i, j]    = sum_g talk[h, g] p_g[i, j]
+//   o_h[i]       = gate_h[i] * sum_j w_h[i, j] v_kv(h)[j],    gate = sigmoid(g_h[i]) elementwise (optional)
+//
+// A mixed weight needs every head's finished statistics, so the keys are walked twice.  MODE 1 forms each head's raw
+// scores and leaves the maximum and the sum of every (work item, row, head) in `stats`; no wave needs another's
+// scores there.  MODE 2 folds the statistics of all runs of its row block (with the sink), forms the raw scores
+// again, turns them into finished weights, exchanges those through LDS, mixes them and adds O^T += V^T W^T: nothing
+// is rescaled afterwards, so the runs of a row block simply add up (talk_sum_kernel, which also applies the gate).
 // Scores, weights, statistics and accumulators are float; products read the compute dtype T.
 // Keys a request does not hold (beyond its length, pages a window has released) enter as zeros and
 // are masked; their values are replaced by zeros before the product.
@@ -67,12 +79,18 @@ __device__ __forceinline__ typename Atom<T>::vec_t load_or_zero(const T* p, bool
   return ok ? v : Atom<T>::zero();
 }
 
-template <typename T>
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+constexpr int kStatRows = 16;   // rows of a work item in `stats` (also for decoded tokens, which use row 0)
+
+// MODE 0: the heads' scores are mixed before the softmax.  MODE 1 / 2: the two passes that mix the heads' weights.
+template <typename T, int MODE>
 __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ k_pages, const T* __restrict__ v_pages, int page_size,
     const int* __restrict__ table, int table_stride, const SeqMeta* __restrict__ seqs, const int* __restrict__ blocks,
     const float* __restrict__ talk, float scale, int window, int keep_first, T* __restrict__ out, long ldo,
-    float* __restrict__ part, int part_rows) {
+    float* __restrict__ part, int part_rows, const float* __restrict__ sink, float* __restrict__ stats,
+    const float* __restrict__ gate, long ldg) {
   constexpr int VEC = Atom<T>::VEC, KC = Atom<T>::KCHUNK;
   constexpr int KCH = (D + KC - 1) / KC;  // chunks of a key (lanes beyond D in the last one bring zeros)
   __shared__ f32x4 raw_s[H][2][64];  // [head][half of the tile][lane]: the lane's four keys of that half
@@ -111,6 +129,25 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 
   const int per_run = (n_tiles + n_runs - 1) / n_runs;
   const int step_end = min(n_tiles, (run + 1) * per_run);
+
+  // MODE 2: every own head's finished maximum and the inverse of its finished sum, folded over the runs of this row
+  // block in ascending order (their work items follow each other), with the sink
+  float m_all[HPW], inv_all[HPW];
+  if constexpr (MODE == 2) {
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+      const int h = w * HPW + x;
+      const float* st = stats + (((long)(blockIdx.x - run) * kStatRows + (row_ok ? l16 : 0)) * H + h) * 2;
+      const long stride = (long)kStatRows * H * 2;
+      float top = sink ? sink[h] : kNegSentinel;
+      for (int k = 0; k < n_runs; ++k) top = fmaxf(top, st[k * stride]);
+      float total = 0.f;
+      for (int k = 0; k < n_runs; ++k) total = total + st[k * stride + 1] * softmax_exp<T>(st[k * stride] - top);
+      if (sink) total = total + softmax_exp<T>(sink[h] - top);
+      m_all[x] = top;
+      inv_all[x] = row_ok && total > 0.f ? 1.0f / total : 0.f;
+    }
+  }
 
   // A tile's keys are requested while the tile before it is worked on: its addresses (page and slot of the
   // lane's key of each half as a row of K, and of its four keys as columns of V^T) and the key vectors of the
@@ -175,6 +212,7 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
       for (int i = 0; i < 4; ++i) v_ok[half][i] = now.v_ok[half][i];
     }
     // -- 1. transposed raw scores of the wave's own heads ------------------------------------
+    f32x4 own[MODE == 1 ? HPW : 1][2];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -193,13 +231,21 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
                            load_or_zero<T>(q_row + h * D + (in ? c * KC + VEC * quad : 0), row_ok && in));
             }
           }
-          raw_s[h][half][lane] = f32x4{s[0] * scale, s[1] * scale, s[2] * scale, s[3] * scale};
+          if constexpr (MODE == 0) {
+            raw_s[h][half][lane] = f32x4{s[0] * scale, s[1] * scale, s[2] * scale, s[3] * scale};
+          } else if constexpr (MODE == 1) {
+            own[xg * SH + xs][half] = f32x4{s[0] * scale, s[1] * scale, s[2] * scale, s[3] * scale};
+          } else {   // the head's finished weights (of keys that the row does not see as well: the mask follows the mixing)
+            f32x4 p;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = softmax_exp<T>(s[i] * scale - m_all[xg * SH + xs]) * inv_all[xg * SH + xs];
+            raw_s[h][half][lane] = p;
+          }
         }
       }
     }
     if (step + 1 < step_end) request(step + 1, now);  // (the products above have taken this tile's keys)
-    lds_barrier();
-    // -- 2. mix, mask, online softmax ---------------------------------------------------------------
+    // what a row sees of this tile
     bool see[2][4];
 #pragma unroll
     for (int half = 0; half < 2; ++half)
@@ -208,6 +254,30 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
         const int key = key0 + 16 * half + 4 * quad + i;
         see[half][i] = row_ok && key <= my_pos && (my_pos - key < window || key < keep_first);
       }
+    if constexpr (MODE == 1) {
+      // the statistics of the own heads' raw scores; nothing is exchanged and no value is read
+#pragma unroll
+      for (int x = 0; x < HPW; ++x) {
+        float top = kNegSentinel;
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) top = fmaxf(top, see[half][i] ? own[x][half][i] : kNegSentinel);
+        top = quad16_max(top);
+        const float m_new = fmaxf(m_run[x], top);
+        float sum = 0.f;
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sum = sum + (see[half][i] ? softmax_exp<T>(own[x][half][i] - m_new) : 0.f);
+        sum = quad16_sum(sum);
+        l_run[x] = l_run[x] * softmax_exp<T>(m_run[x] - m_new) + sum;
+        m_run[x] = m_new;
+      }
+      continue;
+    }
+    lds_barrier();
+    // -- 2. mix, mask, online softmax ---------------------------------------------------------------
     // every head's raw scores are read once and go into all of the wave's own heads
     float mixed[HPW][2][4];
 #pragma unroll
@@ -216,22 +286,38 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mixed[x][half][i] = 0.f;
+    // (the second pass of mixed weights holds more than the first way of mixing: it reads four heads at a time, so
+    // that the reads of all heads are not in registers together)
+    constexpr int OU = (MODE == 2 && H > 4) ? 4 : H;
+#pragma unroll 1
+    for (int o0 = 0; o0 < H; o0 += OU) {
 #pragma unroll
-    for (int o = 0; o < H; ++o) {
-      const f32x4 r0 = raw_s[o][0][lane], r1 = raw_s[o][1][lane];
+      for (int oo = 0; oo < OU; ++oo) {
+        const int o = o0 + oo;
+        if (o >= H) break;
+        const f32x4 r0 = raw_s[o][0][lane], r1 = raw_s[o][1][lane];
 #pragma unroll
-      for (int x = 0; x < HPW; ++x) {
-        const float weight = talk_s[(w * HPW + x) * H + o];
+        for (int x = 0; x < HPW; ++x) {
+          const float weight = talk_s[(w * HPW + x) * H + o];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {  // (fused multiply-adds, written as such: this loop is the kernel's vector work)
-          mixed[x][0][i] = fmaf(weight, r0[i], mixed[x][0][i]);
-          mixed[x][1][i] = fmaf(weight, r1[i], mixed[x][1][i]);
+          for (int i = 0; i < 4; ++i) {  // (fused multiply-adds, written as such: this loop is the kernel's vector work)
+            mixed[x][0][i] = fmaf(weight, r0[i], mixed[x][0][i]);
+            mixed[x][1][i] = fmaf(weight, r1[i], mixed[x][1][i]);
+          }
         }
       }
     }
     float shrink[HPW];
 #pragma unroll
     for (int x = 0; x < HPW; ++x) {     // the scores become the weights, in place
+      if constexpr (MODE == 2) {        // (they are weights already, and finished; a weight of a key that is not seen
+        shrink[x] = 1.0f;               //  may be anything, also no number: it is replaced, never multiplied)
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mixed[x][half][i] = see[half][i] ? mixed[x][half][i] : 0.f;
+        continue;
+      }
       float top = kNegSentinel;
 #pragma unroll
       for (int half = 0; half < 2; ++half)
@@ -338,6 +424,17 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
     lds_barrier();
   }
   if (!row_ok) return;
+  if constexpr (MODE == 1) {
+    if (quad == 0) {
+#pragma unroll
+      for (int x = 0; x < HPW; ++x) {
+        float* st = stats + (((long)blockIdx.x * kStatRows + l16) * H + w * HPW + x) * 2;
+        st[0] = m_run[x];
+        st[1] = l_run[x];
+      }
+    }
+    return;
+  }
   if (n_runs > 1) {
     // [item][row][head][DV + 2]: the unnormalised output, then max and sum (part_rows 1: decoded tokens, row 0 only)
     if (l16 >= part_rows) return;
@@ -349,7 +446,7 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (16 * b + 4 * quad + i < DV) dst[16 * b + 4 * quad + i] = acc[x][b][i];
-      if (quad == 0) {
+      if (MODE == 0 && quad == 0) {
         dst[DV] = m_run[x];
         dst[DV + 1] = l_run[x];
       }
@@ -360,12 +457,40 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
 #pragma unroll
   for (int x = 0; x < HPW; ++x) {
     const int h = w * HPW + x;
-    const float inv = 1.0f / l_run[x];
+    const float inv = MODE == 2 ? 1.0f : 1.0f / l_run[x];
+    const float* g_row = (MODE == 2 && gate) ? gate + (long)(m.q_off + row0 + l16) * ldg + h * DV : nullptr;
 #pragma unroll
     for (int b = 0; b < VB; ++b)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (16 * b + 4 * quad + i < DV) dst[h * DV + 16 * b + 4 * quad + i] = from_f32<T>(acc[x][b][i] * inv);
+      for (int i = 0; i < 4; ++i) {
+        const int c = 16 * b + 4 * quad + i;
+        if (c < DV) {
+          float v = acc[x][b][i] * inv;
+          if (g_row) v = v * sigmoid_f(g_row[c]);
+          dst[h * DV + c] = from_f32<T>(v);
+        }
+      }
+  }
+}
+
+// The runs of a row block whose weights were mixed after the softmax: their outputs add up, in ascending order, and
+// the gate multiplies the sum.  One workgroup a (fold item, head, row), as talk_combine_kernel.
+template <typename T>
+__global__ __launch_bounds__(64) void talk_sum_kernel(const float* __restrict__ part, int part_rows,
+                                                      const int* __restrict__ folds, const float* __restrict__ gate,
+                                                      long ldg, T* __restrict__ out, long ldo) {
+  const int first = folds[4 * blockIdx.x], n_runs = folds[4 * blockIdx.x + 1];
+  const int row0 = folds[4 * blockIdx.x + 2], rows = folds[4 * blockIdx.x + 3];
+  const int h = blockIdx.y;
+  const long stride = (long)part_rows * H * (DV + 2);  // from a run to the next
+  for (int r = blockIdx.z; r < rows; r += gridDim.z) {
+    const float* mine = part + (((long)first * part_rows + r) * H + h) * (DV + 2);
+    for (int c = threadIdx.x; c < DV; c += 64) {
+      float sum = 0.f;
+      for (int k = 0; k < n_runs; ++k) sum = sum + mine[k * stride + c];
+      if (gate) sum = sum * sigmoid_f(gate[(long)(row0 + r) * ldg + (long)h * DV + c]);
+      out[(long)(row0 + r) * ldo + h * DV + c] = from_f32<T>(sum);
+    }
   }
 }
 
@@ -416,7 +541,13 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
                                  int page_size, const int* table, int table_stride, const void* seqs,
                                  const int* blocks, int n_blocks, const float* talk, float scale, int window,
                                  int keep_first, void* out, long ldo, const int* folds, int n_folds, float* part,
-                                 int part_rows, void* stream) {
+                                 int part_rows, int mix_weights, const float* sink, float* stats, const float* gate,
+                                 long ldg, void* stream) {
+  // mix_weights: the heads' weights are mixed after each head's own softmax (two passes; stats: n_blocks * 16 * H * 2
+  // floats of scratch), with an optional sink [H] in every head's softmax and an optional gate (float [T][ldg], H
+  // heads of DV logits) on the output; else the scores are mixed before the softmax, and sink and gate must be null.
+  LS_REQUIRE(mix_weights ? stats != nullptr : (!sink && !gate), "talk_attention: a sink and a gate come with mixed weights");
+  LS_REQUIRE(!gate || ldg >= (long)H * DV, "talk_attention: the gate's rows are too short");
   LS_REQUIRE(n_folds >= 0 && (n_folds == 0 || (part && folds && (part_rows == 1 || part_rows == 16))),
              "talk_attention: %d fold items need partial results of 1 or 16 rows", n_folds);
   LS_REQUIRE(n_blocks > 0 && q && k_pages && v_pages && table && seqs && blocks && talk && out, "talk_attention: null operand");
@@ -427,25 +558,35 @@ extern "C" int ls_talk_attention(int dtype, const void* q, long ldq, const void*
                  reinterpret_cast<uintptr_t>(v_pages) % 16 == 0,
              "talk_attention: operands must be 16-byte aligned");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define LS_TALK_PASS(T_, MODE_)                                                                                        \
+  hipLaunchKernelGGL((talk_attention_kernel<T_, MODE_>), dim3(n_blocks), dim3(64 * NW), 0, s, (const T_*)q, ldq,       \
+                     (const T_*)k_pages, (const T_*)v_pages, page_size, table, table_stride, (const SeqMeta*)seqs,     \
+                     blocks, talk, scale, window, keep_first, (T_*)out, ldo, part, part_rows, sink, stats, gate, ldg)
+#define LS_TALK(T_)                                                                                                    \
+  do {                                                                                                                 \
+    if (mix_weights) {                                                                                                 \
+      LS_TALK_PASS(T_, 1);                                                                                             \
+      LS_TALK_PASS(T_, 2);                                                                                             \
+      if (n_folds > 0)                                                                                                 \
+        hipLaunchKernelGGL(talk_sum_kernel<T_>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, folds,   \
+                           gate, ldg, (T_*)out, ldo);                                                                  \
+    } else {                                                                                                           \
+      LS_TALK_PASS(T_, 0);                                                                                             \
+      if (n_folds > 0)                                                                                                 \
+        hipLaunchKernelGGL(talk_combine_kernel<T_>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows,      \
+                           folds, (T_*)out, ldo);                                                                      \
+    }                                                                                                                  \
+  } while (0)
   if (dtype == kF32) {
     LS_REQUIRE(ldq % 4 == 0, "talk_attention: query rows must be 16-byte aligned");
-    hipLaunchKernelGGL(talk_attention_kernel<float>, dim3(n_blocks), dim3(64 * NW), 0, s, (const float*)q, ldq,
-                       (const float*)k_pages, (const float*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (float*)out, ldo, part, part_rows);
-    if (n_folds > 0)
-      hipLaunchKernelGGL(talk_combine_kernel<float>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, folds,
-                         (float*)out, ldo);
+    LS_TALK(float);
   } else if (dtype == kBF16) {
     LS_REQUIRE(ldq % 8 == 0, "talk_attention: query rows must be 16-byte aligned");
-    hipLaunchKernelGGL(talk_attention_kernel<bf16_t>, dim3(n_blocks), dim3(64 * NW), 0, s, (const bf16_t*)q, ldq,
-                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_size, table, table_stride,
-                       (const SeqMeta*)seqs, blocks, talk, scale, window, keep_first, (bf16_t*)out, ldo, part,
-                       part_rows);
-    if (n_folds > 0)
-      hipLaunchKernelGGL(talk_combine_kernel<bf16_t>, dim3(n_folds, H, part_rows), dim3(64), 0, s, part, part_rows, folds,
-                         (bf16_t*)out, ldo);
+    LS_TALK(bf16_t);
   } else {
     return fail("talk_attention: unknown dtype %d", dtype);
   }
+#undef LS_TALK
+#undef LS_TALK_PASS
   return check_launch("talk_attention");
 }

@@ -65,6 +65,13 @@ class Model:
         for run in self.schedule:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"the schedule names layer {run.layer}, the model has {len(self.layers)}")
+            if (run.state is None) != (self.layers[run.layer].state_spec() is None):
+                raise ValueError(f"layer {run.layer} keeps state of its own exactly when its schedule entry names a unit for it")
+        # an embedding that keeps something per request (the token before) finds its unit here
+        embedding_spec = self.embedding.state_spec() if hasattr(self.embedding, "state_spec") else None
+        if (self.spec.embedding_state is None) != (embedding_spec is None):
+            raise ValueError("the embedding keeps state exactly when the model names a cache unit for it")
+        self.embedding.state_unit = self.spec.embedding_state
         self.workspace = Workspace(rt.device)
         self.use_graphs = os.environ.get("LOCKSTEP_NO_GRAPHS", "") in ("", "0")
         # debugging aid: every replayed decode step is also run eagerly and the logits compared bit for bit
@@ -130,6 +137,10 @@ class Model:
             mixer = self.layers[run.layer].mixer
             if run.writes_cache and mixer is not None:
                 units[run.cache] = mixer.cache_spec()
+            if run.state is not None:
+                units[run.state] = self.layers[run.layer].state_spec()
+        if self.spec.embedding_state is not None:
+            units[self.spec.embedding_state] = self.embedding.state_spec()
         return units
 
     def make_cache(self, num_pages: int, page_size: int = 16, max_requests: int = 64,

@@ -92,6 +92,9 @@ class RunKinds:
             tensors = dict(device_constants(layer))
             for i, t in enumerate(cache.unit_tensors(run.cache)):
                 tensors[f"cache[{i}]"] = t
+            if getattr(run, "state", None) is not None:
+                for i, t in enumerate(cache.unit_tensors(run.state)):
+                    tensors[f"state[{i}]"] = t
             group = cache.unit_place.get(run.cache, (None,))[0]
             self.addresses.append({name: (t.data_ptr(), t.numel() * t.element_size()) for name, t in tensors.items()})
             if not repeatable_tree(layer):

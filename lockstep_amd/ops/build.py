@@ -253,10 +253,12 @@ def build_attention_mutants(head_dim: int, force: bool = False) -> Path:
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 MUTANT_HEAD_DIMS = (16, 32, 128)     # the head sizes of the tests that use the controls
 #: (query heads, kv heads, key size, value size) of the talking-heads attention the tests and measurements use
-DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128))
+DEFAULT_TALKING_SHAPES = ((4, 2, 32, 16), (6, 3, 48, 24), (3, 1, 24, 40), (2, 2, 16, 16), (16, 8, 128, 128),
+                          (4, 2, 24, 24), (6, 1, 16, 12), (1, 1, 16, 16), (2, 1, 16, 16))
 #: (key size, value size) of the sink attention the tests and measurements use
 DEFAULT_SINK_SHAPES = ((16, 16), (32, 16), (24, 24), (40, 40), (32, 32), (24, 6), (128, 128),
-                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (48, 32), (192, 128), (320, 256))
+                       (24, 40), (40, 32), (48, 36), (16, 6), (16, 8), (24, 8), (32, 48), (16, 24), (24, 16), (48, 32), (192, 128), (320, 256),
+                       (16, 40), (40, 24))
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True, mutants: bool = True,

@@ -814,13 +814,17 @@ class Kernels:
     def talk_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
                        page_size: int, table, seqs, blocks: torch.Tensor, n_blocks: int, talk: torch.Tensor,
                        scale: float, window: int, keep_first: int, out: torch.Tensor, folds: torch.Tensor | None = None,
-                       n_folds: int = 0, part: torch.Tensor | None = None, part_rows: int = 16) -> None:
+                       n_folds: int = 0, part: torch.Tensor | None = None, part_rows: int = 16,
+                       mix_weights: bool = False, sink=None, stats: torch.Tensor | None = None, gate=None) -> None:
         """Talking-heads attention of the step's queries ``q [T, heads*dim]`` over the paged cache; ``blocks``
         lists ``n_blocks`` work items of four ints (request of the step, block of 16 of its rows, run, runs);
         ``talk [heads, heads]``.  A row block whose visible keys are dealt to several work items (runs > 1) has a
         fold item of four ints in ``folds`` (first work item, runs, first packed row, rows); their results wait in
         ``part`` (float32, ``n_blocks * part_rows * heads * (vdim + 2)`` elements; ``part_rows`` 16, or 1 for a step
-        of single decoded tokens) until a second launch has folded them."""
+        of single decoded tokens) until a second launch has folded them.  ``mix_weights``: the heads' weights are
+        mixed after each head's own softmax instead of their scores before it (``stats``: float32 scratch of
+        ``n_blocks * 16 * heads * 2`` elements), with ``sink [heads]`` (float32 or None) in every head's denominator
+        and ``gate`` (float32 rows of ``heads*vdim`` logits or None) whose sigmoid multiplies the output."""
         lib = self.talking_lib(heads, kv_heads, dim, vdim)
         _rows_ok(q, "talk_attention q"); _rows_ok(out, "talk_attention out")
         if not (q.dtype in DTYPE_CODE and out.dtype == q.dtype and q.shape[1] == heads * dim
@@ -838,13 +842,27 @@ class Kernels:
         self._f32_vector(talk, heads * heads, "talk_attention talk")
         if not (window > 0 and keep_first >= 0):
             raise KernelError(f"talk_attention window {window} / kept first tokens {keep_first}")
+        ldg = 0
+        if mix_weights:
+            if not (stats is not None and stats.is_cuda and stats.dtype == torch.float32 and stats.is_contiguous()
+                    and stats.numel() >= n_blocks * 16 * heads * 2):
+                raise KernelError("talk_attention stats: float32 with 32 * heads elements a work item")
+            if sink is not None:
+                self._f32_vector(sink, heads, "talk_attention sink")
+            if gate is not None:
+                _rows_ok(gate, "talk_attention gate")
+                if not (gate.dtype == torch.float32 and gate.shape[0] >= q.shape[0] and gate.shape[1] == heads * vdim):
+                    raise KernelError(f"talk_attention gate must be float32 [>= {q.shape[0]}, {heads * vdim}]")
+                ldg = gate.stride(0)
+        elif sink is not None or gate is not None:
+            raise KernelError("talk_attention: a sink and a gate come with mixed weights only")
         if n_blocks == 0:
             return
         self._launch(lib, lib.ls_talk_attention, (
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
             _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(blocks), c_int(n_blocks), _ptr(talk), c_float(scale),
             c_int(window), c_int(keep_first), _ptr(out), c_long(out.stride(0)), _ptr(folds), c_int(n_folds), _ptr(part),
-            c_int(part_rows), _stream()))
+            c_int(part_rows), c_int(int(bool(mix_weights))), _ptr(sink), _ptr(stats), _ptr(gate), c_long(ldg), _stream()))
 
     LINREC_HGRN2, LINREC_RETENTION = 0, 1
 
@@ -901,9 +919,13 @@ class Kernels:
             c_int(positions), c_int(max_pos), _ptr(tok_pos), _ptr(seqs), c_int(n_seqs), _ptr(state), _ptr(gates),
             _ptr(out), c_long(out.stride(0)), _stream()))
 
-    def head_norm_gate(self, x: torch.Tensor, heads: int, vdim: int, weight, gate, eps: float, out: torch.Tensor) -> None:
+    def head_norm_gate(self, x: torch.Tensor, heads: int, vdim: int, weight, gate, eps: float, out: torch.Tensor,
+                       gate_act: str = "silu") -> None:
         """Per (token, head): ``x / sqrt(mean(x^2) + eps)`` over the head's ``vdim`` values, times ``weight
-        [vdim]`` and ``silu(gate)`` (float32 rows like ``x``) where given; ``x`` float32 ``[T, heads*vdim]``."""
+        [vdim]`` and ``silu(gate)`` or, with ``gate_act = "sigmoid"``, ``sigmoid(gate)`` (float32 rows like ``x``)
+        where given; ``x`` float32 ``[T, heads*vdim]``."""
+        if gate_act not in ("silu", "sigmoid"):
+            raise KernelError(f"head_norm_gate: the gate's activation is silu or sigmoid, got {gate_act!r}")
         _rows_ok(x, "head_norm_gate x"); _rows_ok(out, "head_norm_gate out")
         if not (x.dtype == torch.float32 and x.shape[1] == heads * vdim and out.shape == x.shape and out.dtype in DTYPE_CODE):
             raise KernelError("head_norm_gate reads float32 [T, heads*vdim] and writes the same shape")
@@ -920,7 +942,8 @@ class Kernels:
         lib = self.mixers_lib()
         self._launch(lib, lib.ls_head_norm_gate, (
             c_int(DTYPE_CODE[out.dtype]), _ptr(x), c_long(x.stride(0)), c_int(x.shape[0]), c_int(heads), c_int(vdim),
-            _ptr(weight), _ptr(gate), c_long(ldg), c_float(eps), _ptr(out), c_long(out.stride(0)), _stream()))
+            _ptr(weight), _ptr(gate), c_long(ldg), c_int(int(gate_act == "sigmoid")), c_float(eps), _ptr(out),
+            c_long(out.stride(0)), _stream()))
 
 
     # -- attention with a sink, and what comes before it --------------------------------------
@@ -954,14 +977,15 @@ class Kernels:
     def qkv_post(self, raw: torch.Tensor, n_tokens: int, heads: int, kv_heads: int, dim: int, vdim: int, bias, q_norm,
                  k_norm, eps: float, cos, sin, rot: int, neighbours: bool, max_pos: int, tok_seq, tok_pos, seqs, table,
                  q_out: torch.Tensor, k_pages, v_pages, page_size: int, keys_are_values: bool = False,
-                 key_pad: int | None = None, per_head: bool = False) -> None:
+                 key_pad: int | None = None, per_head: bool = False, head_weights: bool = False) -> None:
         """Post pass of the fused projection ``raw`` (float32, ``q | k | v | ...``; no ``v`` with
         ``keys_are_values``, where the biased, unnormalised keys are stored as the values): biases, a
         root-mean-square norm over the whole of q and of k with the weights ``q_norm`` / ``k_norm``, rotation of
         the first ``rot`` dimensions of each head in pairs ``(i, i + rot/2)`` or of ``neighbours``, queries to
         ``q_out``, keys and values to their pages.  ``key_pad``: the size of a head in ``q_out`` and in the key
         pages where it exceeds ``dim`` (zeros beyond ``dim``).  ``per_head``: every head of q and of k is divided
-        by its own root mean square over ``dim`` (``eps`` inside the root, no weights) instead."""
+        by its own root mean square over ``dim`` (``eps`` inside the root, no weights) instead; with
+        ``head_weights`` as well, then multiplied by ``q_norm`` / ``k_norm`` of ``dim`` elements, which all heads share."""
         _rows_ok(raw, "qkv_post raw"); _rows_ok(q_out, "qkv_post q_out")
         key_pad = dim if key_pad is None else key_pad
         width = heads * dim + kv_heads * dim + (0 if keys_are_values else kv_heads * vdim)
@@ -975,10 +999,13 @@ class Kernels:
             self._f32_vector(bias, width, "qkv_post bias")
         if (q_norm is None) != (k_norm is None):
             raise KernelError("qkv_post normalises both q and k or neither")
+        if head_weights and not (per_head and q_norm is not None):
+            raise KernelError("qkv_post: weights that the heads share belong to a norm a head, and both are needed")
         if q_norm is not None:
-            self._f32_vector(q_norm, heads * dim, "qkv_post q_norm"); self._f32_vector(k_norm, kv_heads * dim, "qkv_post k_norm")
-        if per_head and (q_norm is not None or not eps > 0):
-            raise KernelError("qkv_post: a norm a head takes no weights and needs a positive eps")
+            self._f32_vector(q_norm, dim if head_weights else heads * dim, "qkv_post q_norm")
+            self._f32_vector(k_norm, dim if head_weights else kv_heads * dim, "qkv_post k_norm")
+        if per_head and ((q_norm is not None and not head_weights) or not eps > 0):
+            raise KernelError("qkv_post: a norm a head takes no weights, or one vector for all heads, and needs a positive eps")
         positions = self._rotation_tables(cos, sin, rot, max_pos)
         self._paged_ok(k_pages, v_pages, table, q_out.dtype, kv_heads, page_size, key_pad, vdim)
         if not (max_pos // page_size < table.shape[1]):
@@ -991,7 +1018,7 @@ class Kernels:
         lib = self.mixers_lib()
         self._launch(lib, lib.ls_qkv_post, (
             c_int(DTYPE_CODE[q_out.dtype]), _ptr(raw), c_long(raw.stride(0)), c_int(n_tokens), c_int(heads),
-            c_int(kv_heads), c_int(dim), c_int(key_pad), c_int(vdim), c_int(int(keys_are_values)), c_int(int(per_head)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
+            c_int(kv_heads), c_int(dim), c_int(key_pad), c_int(vdim), c_int(int(keys_are_values)), c_int(2 if head_weights else int(per_head)), _ptr(bias), _ptr(q_norm), _ptr(k_norm),
             c_float(eps), _ptr(cos), _ptr(sin), c_int(rot), c_int(int(neighbours)), c_int(positions), c_int(max_pos),
             _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table), c_int(table.shape[1]), _ptr(q_out),
             c_long(q_out.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size), _stream()))
@@ -999,12 +1026,13 @@ class Kernels:
     def sink_attention(self, q: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, k_pages, v_pages,
                        page_size: int, table, seqs, items: torch.Tensor, n_items: int, row_tiles: int, scale: float,
                        window: int, chunk: int, sink, dist_bias, gate, out: torch.Tensor,
-                       folds: torch.Tensor | None = None, n_folds: int = 0, part: torch.Tensor | None = None) -> None:
+                       folds: torch.Tensor | None = None, n_folds: int = 0, part: torch.Tensor | None = None,
+                       keep_first: int = 0) -> None:
         """Attention of the step's queries ``q [T, heads*dim]`` over the paged cache with a sink in the softmax.
         ``items``: ``n_items`` work items of four ints (request of the step, block of ``16 * row_tiles`` of its
         rows, run, runs); ``row_tiles`` 1, 2 or 4, or 0 for a step of single decoded tokens, or ``SINK_STAGED`` for
         the kernel that stages key tiles in LDS (blocks of ``sink_staged_rows`` rows).  ``window`` /
-        ``chunk``: 0 for none.  ``sink [heads]`` float32 or None; ``dist_bias [heads, distances]`` float32 or
+        ``chunk``: 0 for none; ``keep_first``: with a window, the first that many tokens stay visible.  ``sink [heads]`` float32 or None; ``dist_bias [heads, distances]`` float32 or
         None (its last column serves every larger distance); ``gate``: float32 rows of ``heads*vdim`` logits
         whose sigmoid multiplies the output, or None.  Row blocks whose keys are dealt to several work items
         have a fold item in ``folds`` (first work item, runs, first packed row, rows) and their results wait in
@@ -1047,12 +1075,14 @@ class Kernels:
             ldg = gate.stride(0)
         if not (window >= 0 and chunk >= 0):
             raise KernelError(f"sink_attention window {window} / chunk {chunk}")
+        if not (keep_first >= 0 and (keep_first == 0 or (window > 0 and chunk == 0))):
+            raise KernelError(f"sink_attention: {keep_first} kept first tokens need a window and no chunks")
         if n_items == 0:
             return
         self._launch(lib, lib.ls_sink_attention, (
             c_int(DTYPE_CODE[q.dtype]), _ptr(q), c_long(q.stride(0)), _ptr(k_pages), _ptr(v_pages), c_int(page_size),
             _ptr(table), c_int(table.shape[1]), _ptr(seqs), _ptr(items), c_int(n_items), c_int(row_tiles), c_int(heads),
-            c_int(kv_heads), c_float(scale), c_int(window), c_int(chunk), _ptr(sink), _ptr(dist_bias), c_int(n_dist),
+            c_int(kv_heads), c_float(scale), c_int(window), c_int(chunk), c_int(keep_first), _ptr(sink), _ptr(dist_bias), c_int(n_dist),
             _ptr(gate), c_long(ldg), _ptr(out), c_long(out.stride(0)), _ptr(folds), c_int(n_folds), _ptr(part),
             c_int(part_rows), _stream()))
 
@@ -1080,12 +1110,16 @@ class Kernels:
             raise KernelError(f"{name} must be int32 with at least {n} elements on the GPU")
 
     def experts_route(self, logits: torch.Tensor, bias, top: int, rows_a_tile: int, expert: torch.Tensor,
-                      weight: torch.Tensor, order: torch.Tensor, tiles: torch.Tensor, counts: torch.Tensor) -> None:
+                      weight: torch.Tensor, order: torch.Tensor, tiles: torch.Tensor, counts: torch.Tensor,
+                      scoring: str = "softmax") -> None:
         """From router ``logits [T, E]`` (float32) and ``bias [E]``: every token's ``top`` experts (largest logit
         first, the lower index wins a tie) into ``expert [T, top]``, the softmax over the chosen logits into
         ``weight [T, top]``; the pairs ``token * top + choice`` sorted by expert into ``order``, and every
-        expert's pairs cut into ``tiles [capacity, 4]`` (expert or -1, first place in ``order``, rows, 0)."""
+        expert's pairs cut into ``tiles [capacity, 4]`` (expert or -1, first place in ``order``, rows, 0).
+        ``scoring = "sigmoid"``: every chosen expert weighs the sigmoid of its own logit instead, not renormalised."""
         _rows_ok(logits, "experts_route logits")
+        if scoring not in ("softmax", "sigmoid"):
+            raise KernelError(f"experts_route: scoring is softmax or sigmoid, got {scoring!r}")
         t, e = logits.shape
         if not (logits.dtype == torch.float32 and 0 < top <= min(e, self.experts_max_top())):
             raise KernelError(f"experts_route: float32 logits and 1 <= top <= {min(e, self.experts_max_top())}, got {top}")
@@ -1101,17 +1135,21 @@ class Kernels:
         lib = self.experts_lib()
         self._launch(lib, lib.ls_experts_route, (
             _ptr(logits), c_long(logits.stride(0)), _ptr(bias), c_int(t), c_int(e), c_int(top), c_int(rows_a_tile),
-            _ptr(expert), _ptr(weight), _ptr(order), _ptr(tiles), c_int(cap), _ptr(counts), _stream()))
+            _ptr(expert), _ptr(weight), _ptr(order), _ptr(tiles), c_int(cap), _ptr(counts), c_int(int(scoring == "sigmoid")),
+            _stream()))
 
     def experts_apply(self, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, top: int,
                       rows_a_tile: int, order: torch.Tensor, tiles: torch.Tensor, weight: torch.Tensor, limit: float,
-                      alpha: float, act: torch.Tensor, partials: torch.Tensor, shift: float = 1.0) -> None:
+                      alpha: float, act: torch.Tensor, partials: torch.Tensor, shift: float = 1.0,
+                      weigh_input: bool = False) -> None:
         """``partials[k][t] = weight[t, k] * down_e(act(gate_e x[t], up_e x[t]))`` for every token's ``k``-th
         expert ``e``, with the clamped gated unit of ``glu_clamped`` as activation (``min(g, limit) sigmoid(alpha
         min(g, limit)) (clamp(u, -limit, limit) + shift)``; an infinite ``limit``, ``alpha`` 1 and ``shift`` 0 are the
         plain unit ``silu(g) u``).  ``w_gate``, ``w_up``
         ``[E, F, K]``, ``w_down [E, N, F]`` in the compute dtype; ``act``: scratch ``[T * top, F]`` of the
-        compute dtype; ``partials [top, T, N]`` float32; the routing as ``experts_route`` left it."""
+        compute dtype; ``partials [top, T, N]`` float32; the routing as ``experts_route`` left it.
+        ``weigh_input``: the weight multiplies the expert's input instead, ``partials[k][t] = down_e(act(w gate_e
+        x[t], w up_e x[t]))``."""
         _rows_ok(x, "experts_apply x"); _rows_ok(act, "experts_apply act")
         t, k = x.shape
         if not (w_gate.dim() == 3 and w_gate.shape == w_up.shape and w_gate.shape[2] == k and w_down.dim() == 3
@@ -1136,7 +1174,7 @@ class Kernels:
             c_int(DTYPE_CODE[x.dtype]), _ptr(x), c_long(x.stride(0)), _ptr(w_gate), _ptr(w_up), _ptr(w_down), c_int(t),
             c_int(e), c_int(top), c_int(k), c_int(f), c_int(n), c_int(rows_a_tile), _ptr(order), _ptr(tiles), c_int(cap),
             _ptr(weight), c_float(limit), c_float(alpha), c_float(shift), _ptr(act), c_long(act.stride(0)), _ptr(partials),
-            _stream()))
+            c_int(int(bool(weigh_input))), _stream()))
 
     def experts_route_table(self, token_ids: torch.Tensor, table: torch.Tensor, experts: int, rows_a_tile: int,
                             expert: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, tiles: torch.Tensor,
@@ -1297,14 +1335,15 @@ class Kernels:
     def delta_max_dim(self) -> int:
         return self._memo(("delta_max_dim",), lambda: int(self.mixers_lib().ls_delta_max_dim()))
 
-    def delta_scratch_floats(self, n_tokens: int, kv_heads: int, heads: int, dim: int, vdim: int) -> int:
+    def delta_scratch_floats(self, n_tokens: int, kv_heads: int, heads: int, dim: int, vdim: int, channel: bool = False) -> int:
         lib = self.mixers_lib()
-        lib.ls_delta_scratch_floats.restype = ctypes.c_long
-        return int(lib.ls_delta_scratch_floats(c_int(n_tokens), c_int(kv_heads), c_int(heads), c_int(dim), c_int(vdim)))
+        entry = lib.ls_delta_scratch_floats_channel if channel else lib.ls_delta_scratch_floats
+        entry.restype = ctypes.c_long
+        return int(entry(c_int(n_tokens), c_int(kv_heads), c_int(heads), c_int(dim), c_int(vdim)))
 
     def delta_rule(self, raw: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int, taps: torch.Tensor, a_log,
                    dt_bias, unit_eps: float, tok_seq, tok_pos, seqs, n_seqs: int, state: torch.Tensor,
-                   scratch: torch.Tensor, out: torch.Tensor) -> None:
+                   scratch: torch.Tensor, out: torch.Tensor, channel_decay: torch.Tensor | None = None) -> None:
         """The gated delta rule over the tokens of every request of the step.  ``raw`` float32 holds the
         projections ``q | k`` (``kv_heads`` heads of ``dim``) ``| v`` (``heads`` of ``vdim``) ``| b | a``
         (``heads`` each); every channel of q, k and v passes a causal convolution with ``taps [channels, M]``
@@ -1312,11 +1351,20 @@ class Kernels:
         the root), q also times ``dim^-1/2``; ``beta = sigmoid(b)``, ``decay = exp(-exp(a_log) softplus(a +
         dt_bias))``; per head ``S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``.  ``state``
         float32 ``[slots, heads*dim*vdim + (M-1)*channels]``: the matrices, then the convolutions' last inputs;
-        read and left for the next step.  ``out`` float32 ``[T, heads*vdim]``."""
+        read and left for the next step.  ``out`` float32 ``[T, heads*vdim]``.  ``channel_decay`` (float32 rows of
+        ``heads*dim`` logits): a decay for every head and key channel instead, ``g = exp(-exp(a_log_h) softplus(logit +
+        dt_bias))`` with ``dt_bias [heads*dim]``, which multiplies the rows of ``S``; ``raw`` then ends with ``b``."""
         _rows_ok(raw, "delta_rule raw"); _rows_ok(out, "delta_rule out")
         t = raw.shape[0]
         channels = 2 * kv_heads * dim + heads * vdim
-        if not (raw.dtype == torch.float32 and raw.shape[1] >= channels + 2 * heads and out.dtype == torch.float32
+        chan = channel_decay is not None
+        ldc = 0
+        if chan:
+            _rows_ok(channel_decay, "delta_rule channel_decay")
+            if not (channel_decay.dtype == torch.float32 and channel_decay.shape[0] >= t and channel_decay.shape[1] == heads * dim):
+                raise KernelError(f"delta_rule channel_decay must be float32 [>= {t}, {heads * dim}]")
+            ldc = channel_decay.stride(0)
+        if not (raw.dtype == torch.float32 and raw.shape[1] >= channels + (1 if chan else 2) * heads and out.dtype == torch.float32
                 and tuple(out.shape) == (t, heads * vdim)):
             raise KernelError("delta_rule reads and writes float32 rows, out [T, heads*vdim]")
         if not (heads % kv_heads == 0 and dim <= self.delta_max_dim()):
@@ -1325,12 +1373,13 @@ class Kernels:
                 and taps.shape[0] == channels and taps.shape[1] >= 1):
             raise KernelError(f"delta_rule taps must be float32 [{channels}, M]")
         m = taps.shape[1]
-        self._f32_vector(a_log, heads, "delta_rule a_log"); self._f32_vector(dt_bias, heads, "delta_rule dt_bias")
+        self._f32_vector(a_log, heads, "delta_rule a_log")
+        self._f32_vector(dt_bias, heads * dim if chan else heads, "delta_rule dt_bias")
         if not (state.is_cuda and state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2
                 and state.shape[1] == heads * dim * vdim + (m - 1) * channels):
             raise KernelError(f"delta_rule state must be float32 [slots, {heads * dim * vdim + (m - 1) * channels}]")
         if not (scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous()
-                and scratch.numel() >= self.delta_scratch_floats(t, kv_heads, heads, dim, vdim)):
+                and scratch.numel() >= self.delta_scratch_floats(t, kv_heads, heads, dim, vdim, chan)):
             raise KernelError("delta_rule scratch: float32 of delta_scratch_floats elements")
         for name, v in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
             if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous() and v.numel() >= t):
@@ -1342,6 +1391,60 @@ class Kernels:
             _ptr(raw), c_long(raw.stride(0)), c_int(t), c_int(kv_heads), c_int(heads), c_int(dim), c_int(vdim), c_int(m),
             _ptr(taps), _ptr(a_log), _ptr(dt_bias), c_float(unit_eps), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs),
             c_int(n_seqs), _ptr(state), c_long(state.stride(0)), _ptr(scratch), _ptr(out), c_long(out.stride(0)),
+            _ptr(channel_decay), c_long(ldc), _stream()))
+
+    # -- an embedding with a table of token pairs, and the shift of a sublayer's input by a token -------------
+    def embed_pair(self, tokens: torch.Tensor, tok_seq, tok_pos, seqs, table: torch.Tensor, pairs: torch.Tensor,
+                   mul_prev: int, mul_cur: int, state: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+        """``out[t] = table[tokens[t]] * scale + pairs[(token before * mul_prev + tokens[t] * mul_cur) mod buckets]``
+        as float32 rows, ``buckets = pairs.shape[0] - 1``; a request's first token takes the last row of ``pairs``.
+        ``state`` int32 ``[slots, 1]``: the last token of every request so far, read for the first row of a portion
+        and left as the portion's last token."""
+        if not (tokens.is_cuda and tokens.dtype == torch.int32 and tokens.dim() == 1 and tokens.is_contiguous()):
+            raise KernelError("embed_pair tokens must be a contiguous int32 vector on the GPU")
+        t = tokens.shape[0]
+        _rows_ok(table, "embed_pair table"); _rows_ok(pairs, "embed_pair pairs"); _rows_ok(out, "embed_pair out")
+        if not (table.is_contiguous() and pairs.is_contiguous() and table.dtype in DTYPE_CODE and pairs.dtype == table.dtype
+                and pairs.shape[1] == table.shape[1] and pairs.shape[0] >= 2):
+            raise KernelError("embed_pair tables must be contiguous, of one dtype and one width, the pairs' with two rows or more")
+        if not (out.dtype == torch.float32 and tuple(out.shape) == (t, table.shape[1])):
+            raise KernelError(f"embed_pair out must be float32 [{t},{table.shape[1]}]")
+        if not (state.is_cuda and state.dtype == torch.int32 and state.dim() == 2 and state.stride(1) == 1):
+            raise KernelError("embed_pair state must be int32 [slots, 1] on the GPU")
+        for name, v in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous() and v.numel() >= t):
+                raise KernelError(f"embed_pair {name}: int32, one entry a token")
+        if t == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_embed_pair, (
+            c_int(DTYPE_CODE[table.dtype]), _ptr(tokens), _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(table),
+            c_int(table.shape[0]), _ptr(pairs), c_int(pairs.shape[0] - 1), c_long(mul_prev), c_long(mul_cur), _ptr(state),
+            c_long(state.stride(0)), _ptr(out), c_int(t), c_int(table.shape[1]), c_long(out.stride(0)), c_float(scale),
+            _stream()))
+
+    def token_shift(self, normed: torch.Tensor, mu: torch.Tensor, tok_seq, tok_pos, seqs, state: torch.Tensor,
+                    out: torch.Tensor) -> None:
+        """``out[t] = n[t] + (n[t-1] - n[t]) * mu`` for the float32 rows ``normed`` of the step, ``n[t-1]`` being the row
+        of the same request's token before (zeros at a request's first token); ``state`` float32 ``[slots, width]``
+        holds that row for the first token of a portion and is left as the portion's last row."""
+        _rows_ok(normed, "token_shift normed"); _rows_ok(out, "token_shift out")
+        t, width = normed.shape
+        if not (normed.dtype == torch.float32 and out.dtype in DTYPE_CODE and tuple(out.shape) == (t, width)):
+            raise KernelError("token_shift reads float32 rows and writes rows of the same shape")
+        self._f32_vector(mu, width, "token_shift mu")
+        if not (state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+                and state.shape[1] >= width):
+            raise KernelError(f"token_shift state must be float32 [slots, >= {width}]")
+        for name, v in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous() and v.numel() >= t):
+                raise KernelError(f"token_shift {name}: int32, one entry a token")
+        if t == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_token_shift, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(normed), c_long(normed.stride(0)), _ptr(mu), _ptr(tok_seq), _ptr(tok_pos),
+            _ptr(seqs), _ptr(state), c_long(state.stride(0)), _ptr(out), c_long(out.stride(0)), c_int(t), c_int(width),
             _stream()))
 
 

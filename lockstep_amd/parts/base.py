@@ -208,6 +208,11 @@ class Arrangement(Part):
         or None for a layer that mixes nothing."""
         raise NotImplementedError
 
+    def state_spec(self):
+        """What the arrangement itself keeps per request between steps, beside its mixer's unit: a
+        ``StateSpec`` (the schedule entry's ``state`` then names the unit) or None."""
+        return None
+
     def forward(self, ctx, run, h) -> None:
         raise NotImplementedError
 

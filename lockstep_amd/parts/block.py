@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from .base import Arrangement, PendingAdd, build_part, register_part, takes
+from .base import Arrangement, PendingAdd, StateSpec, WeightSpec, build_part, register_part, takes
 
 
 @register_part("prenorm_residual")
@@ -13,6 +13,12 @@ class PreNormResidual(Arrangement):
     Parameters name the parts' tensor prefixes below the layer's prefix:
     ``mixer_prefix``, ``feed_forward_prefix``, ``mixer_norm_name``,
     ``feed_forward_norm_name``.  A layer without a ``feed_forward`` part is the first half alone.
+
+    ``token_shift`` (optional, a tensor name below the layer's prefix): what the mixer reads, ``n =
+    norm_1(h)``, is replaced by ``n[t] + (n[t-1] - n[t]) * mu`` with the tensor ``mu [width]`` and the
+    unshifted ``n[t-1]`` of the same request's token before (zeros for its first token).  The last
+    ``n`` of a request is kept between steps: the arrangement then has a ``state_spec`` and its
+    schedule entry names a unit for it.
     """
 
     graph_safe = True
@@ -36,6 +42,15 @@ class PreNormResidual(Arrangement):
         self._defer_ff = self.feed_forward is not None and takes(self.feed_forward.forward, "defer")
         self._norm1_pending = takes(self.mixer_norm.forward, "pending")
         self._norm2_pending = self.feed_forward is not None and takes(self.feed_forward_norm.forward, "pending")
+        self.shift_name = p.get("token_shift")
+        self.shift = None
+        self.width = None
+        if self.shift_name:
+            self.width = int(layer_spec.part("mixer_norm")["size"])
+            self._fuse_mixer = False          # (the shift stands between the norm and the mixer)
+
+    def state_spec(self):
+        return StateSpec((self.width,), "float32") if self.shift_name else None
 
     @classmethod
     def weight_specs(cls, layer_spec, prefix: str = ""):
@@ -44,6 +59,9 @@ class PreNormResidual(Arrangement):
         p = layer_spec.arrangement.params
         base = layer_spec.prefix
         out = []
+        if p.get("token_shift"):
+            out.append(WeightSpec(cls.join(base, p["token_shift"]), (int(layer_spec.part("mixer_norm")["size"]),),
+                                  kind="vector", init="unit"))
         wired = [(layer_spec.part("mixer_norm"), p["mixer_norm_name"]), (layer_spec.part("mixer"), p["mixer_prefix"])]
         if layer_spec.has("feed_forward"):
             wired += [(layer_spec.part("feed_forward_norm"), p["feed_forward_norm_name"]),
@@ -67,6 +85,9 @@ class PreNormResidual(Arrangement):
     def load(self, weights, rt) -> None:
         for part in self.parts():
             part.load(weights, rt)
+        if self.shift_name:
+            self.shift = rt.vector(weights.get(self.join(self.layer_spec.prefix, self.shift_name)))
+            rt.kernels.mixers_lib()
 
     #: a step of at most this many tokens lets the consumer's first matrix
     #: product normalise its input itself (one launch less per norm).  Off by
@@ -93,10 +114,14 @@ class PreNormResidual(Arrangement):
             mixed = self._mixer.forward(ctx, run, h, h, accumulate=True, norm=self.mixer_norm)
         else:
             x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
+            # (with a token shift the norm's rows stay in float32, and the shift writes what the mixer reads)
+            n = ctx.buf("block.unshifted", (ctx.n_tokens, h.shape[1]), __import__("torch").float32) if self.shift_name else x
             if pending is not None:
-                self.mixer_norm.forward(ctx, h, x, pending=pending)
+                self.mixer_norm.forward(ctx, h, n, pending=pending)
             else:
-                self.mixer_norm.forward(ctx, h, x)
+                self.mixer_norm.forward(ctx, h, n)
+            if self.shift_name:
+                rt.kernels.token_shift(n, self.shift, ctx.tok_seq, ctx.tok_pos, ctx.seqs, ctx.cache.unit_state(run.state), x)
             if self._defer_mixer:
                 mixed = self._mixer.forward(ctx, run, x, h, accumulate=True, defer=True)
             else:

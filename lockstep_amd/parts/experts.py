@@ -6,6 +6,10 @@ that every token uses.
     w[t, k]   = softmax over the chosen logits alone
     out[t]    = sum_k w[t, k] * expert_chosen(t)[k](x[t])  +  shared(x[t])
 
+With ``score = "sigmoid"`` the weights are the chosen experts' own scores ``sigmoid(z)`` instead, not renormalised
+(the experts with the largest scores are those with the largest logits).  With ``weigh = "input"`` a weight
+multiplies what its expert reads and not what it returns: ``out[t] = sum_k expert_chosen(t)[k](w[t, k] x[t])``.
+
 With ``router = "table"`` there is no router: row ``token id`` of an integer table ``[vocab, top]`` names
 the token's experts (the entries of a row differ) and each weighs ``1 / top``.
 
@@ -37,7 +41,9 @@ class RoutedExperts(FeedForward):
     below ``<prefix>.shared``).  Tensors below the prefix: ``e<i>.gate``, ``e<i>.up`` ``[F, H]``,
     ``e<i>.down`` ``[H, F]`` for every expert ``i``, ``router`` ``[E, H]`` and ``router.b`` ``[E]``.
     ``limit`` None: the plain gated unit with SiLU.  ``router`` ``"table"`` (default ``"linear"``): the
-    tensor ``table`` ``[vocab_size, top]`` (int) instead of the router's, with the parameter ``vocab_size``."""
+    tensor ``table`` ``[vocab_size, top]`` (int) instead of the router's, with the parameter ``vocab_size``.
+    ``score`` (``"softmax"`` over the chosen logits, the default, or ``"sigmoid"`` of each), ``weigh`` (``"output"``,
+    the default, or ``"input"``), ``router_bias`` (default True; False: there is no tensor ``router.b``)."""
 
     graph_safe = True
 
@@ -54,6 +60,12 @@ class RoutedExperts(FeedForward):
         self.tabled = p.get("router", "linear") == "table"
         if p.get("router", "linear") not in ("linear", "table"):
             raise ValueError(f"router {p['router']!r} is not one of linear, table")
+        self.score, self.weigh = p.get("score") or "softmax", p.get("weigh") or "output"
+        self.router_bias = p.get("router_bias", True) is not False
+        if self.score not in ("softmax", "sigmoid") or self.weigh not in ("output", "input"):
+            raise ValueError(f"score {self.score!r} is not softmax or sigmoid, or weigh {self.weigh!r} not output or input")
+        if self.tabled and self.score != "softmax":
+            raise ValueError("experts that a table names have no scores")
         if not 0 < self.top <= self.experts:
             raise ValueError(f"a token cannot use {self.top} of {self.experts} experts")
         if not self.limit > 0:
@@ -75,7 +87,9 @@ class RoutedExperts(FeedForward):
         if p.get("router", "linear") == "table":
             out.append(WeightSpec(f"{prefix}.table", (int(p["vocab_size"]), int(p["top"])), kind="int", init="distinct", free=e))
         else:
-            out += [WeightSpec(f"{prefix}.router", (e, h)), WeightSpec(f"{prefix}.router.b", (e,), kind="vector")]
+            out.append(WeightSpec(f"{prefix}.router", (e, h)))
+            if p.get("router_bias", True) is not False:
+                out.append(WeightSpec(f"{prefix}.router.b", (e,), kind="vector"))
         if p.get("shared") is not None:
             out += part_class(p["shared"].kind).weight_specs(p["shared"], cls.join(prefix, "shared"))
         return out
@@ -98,7 +112,8 @@ class RoutedExperts(FeedForward):
             rt.kernels.experts_lib()
         else:
             self.w_router = rt.matrix(weights.get(f"{self.prefix}.router"))
-            self.b_router = rt.vector(weights.get(f"{self.prefix}.router.b"))
+            self.b_router = rt.vector(weights.get(f"{self.prefix}.router.b")) if self.router_bias else None
+            rt.kernels.experts_lib()
         if not self.tabled and self.top > rt.kernels.experts_max_top():
             raise ValueError(f"{self.top} experts a token exceed the {rt.kernels.experts_max_top()} the routing kernel picks")
         if self.shared is not None:
@@ -128,12 +143,12 @@ class RoutedExperts(FeedForward):
         else:
             logits = ctx.buf("experts.logits", (t, e), torch.float32)
             k.gemm(x, self.w_router, logits, STORE_F32)
-            k.experts_route(logits, self.b_router, top, rows, chosen, share, order, tiles, counts)
+            k.experts_route(logits, self.b_router, top, rows, chosen, share, order, tiles, counts, scoring=self.score)
         slices = top + (1 if self.shared is not None else 0)
         partials = ctx.buf("experts.slices", (slices * t, self.hidden), torch.float32).view(slices, t, self.hidden)
         act = ctx.buf("experts.act", (t * top, self.inter), rt.dtype)
         k.experts_apply(x, self.w_gate, self.w_up, self.w_down, top, rows, order, tiles, share, self.limit, self.alpha,
-                        act, partials[:top], shift=self.shift)
+                        act, partials[:top], shift=self.shift, weigh_input=self.weigh == "input")
         if self.shared is not None:
             self.shared.forward(ctx, x, partials[top], accumulate=False)
         pending = PendingAdd(partials)

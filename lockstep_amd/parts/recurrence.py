@@ -177,6 +177,15 @@ class GatedDelta(Mixer):
     ``v.conv``; ``b``, ``a`` ``[heads, hidden]``; ``A_log``, ``dt_bias`` ``[heads]``; ``g`` ``[heads*vdim,
     hidden]``; ``norm`` ``[vdim]``; ``o``.
 
+    ``decay = "channel"`` (default ``"head"``): one decay for every head and key channel, which multiplies
+    the rows of ``S``: ``g = exp(-exp(A_log_h) softplus(W_a2 (W_a1 h) + dt_bias))``, laid out heads x
+    ``head_dim``, through a bottleneck of ``decay_rank`` (tensors ``a1 [decay_rank, hidden]``, ``a2 [heads *
+    head_dim, decay_rank]``, ``dt_bias [heads * head_dim]`` instead of ``a`` and ``dt_bias [heads]``).
+    ``gate_rank`` (default None): the output gate's logits come through a bottleneck as well, ``W_g2 (W_g1
+    h)`` (tensors ``g1 [gate_rank, hidden]``, ``g2 [heads * vdim, gate_rank]`` instead of ``g``).
+    ``gate_act`` (``"silu"``, the default, or ``"sigmoid"``): what is applied to the gate's logits.
+    A size of -1 for a rank is one that the checkpoint's tensors decide.
+
     The projections are one matrix product stored in float32; convolutions, gates, the recurrence and
     the per-head norm are computed in 32-bit.  A request's state slot holds the matrices and, behind
     them, the last ``taps - 1`` inputs of every convolution channel."""
@@ -190,23 +199,38 @@ class GatedDelta(Mixer):
         self.heads, self.kv_heads = int(p["num_heads"]), int(p["num_kv_heads"])
         self.d, self.dv, self.taps = int(p["head_dim"]), int(p["value_dim"]), int(p["taps"])
         self.eps, self.unit_eps = float(p["eps"]), float(p["unit_eps"])
+        self.decay = p.get("decay") or "head"
+        self.gate_act = p.get("gate_act") or "silu"
+        self.gate_rank = p.get("gate_rank")
+        if self.decay not in ("head", "channel") or self.gate_act not in ("silu", "sigmoid"):
+            raise ValueError(f"decay {self.decay!r} is not head or channel, or gate_act {self.gate_act!r} not silu or sigmoid")
         if min(self.heads, self.kv_heads, self.d, self.dv, self.taps) <= 0 or self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads over {self.kv_heads} query/key heads with sizes {self.d}, {self.dv} "
                              f"and {self.taps} taps are not a gated delta mixer")
         self.channels = 2 * self.kv_heads * self.d + self.heads * self.dv
-        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = self.w_a2 = self.w_g2 = None
 
     @classmethod
     def weight_specs(cls, spec: PartSpec, prefix: str) -> list[WeightSpec]:
         p = spec.params
         h, n, g, d, dv, m = (int(p[key]) for key in ("hidden_size", "num_heads", "num_kv_heads", "head_dim", "value_dim", "taps"))
-        return [WeightSpec(f"{prefix}.q", (g * d, h)), WeightSpec(f"{prefix}.q.conv", (g * d, m), kind="vector", init="unit"),
-                WeightSpec(f"{prefix}.k", (g * d, h)), WeightSpec(f"{prefix}.k.conv", (g * d, m), kind="vector", init="unit"),
-                WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.v.conv", (n * dv, m), kind="vector", init="unit"),
-                WeightSpec(f"{prefix}.b", (n, h)), WeightSpec(f"{prefix}.A_log", (n,), kind="vector"),
-                WeightSpec(f"{prefix}.norm", (dv,), kind="vector", init="norm"), WeightSpec(f"{prefix}.a", (n, h)),
-                WeightSpec(f"{prefix}.dt_bias", (n,), kind="vector"), WeightSpec(f"{prefix}.g", (n * dv, h)),
-                WeightSpec(f"{prefix}.o", (h, n * dv))]
+        out = [WeightSpec(f"{prefix}.q", (g * d, h)), WeightSpec(f"{prefix}.q.conv", (g * d, m), kind="vector", init="unit"),
+               WeightSpec(f"{prefix}.k", (g * d, h)), WeightSpec(f"{prefix}.k.conv", (g * d, m), kind="vector", init="unit"),
+               WeightSpec(f"{prefix}.v", (n * dv, h)), WeightSpec(f"{prefix}.v.conv", (n * dv, m), kind="vector", init="unit"),
+               WeightSpec(f"{prefix}.b", (n, h)), WeightSpec(f"{prefix}.A_log", (n,), kind="vector"),
+               WeightSpec(f"{prefix}.norm", (dv,), kind="vector", init="norm")]
+        if (p.get("decay") or "head") == "channel":
+            rank = int(p["decay_rank"])
+            out += [WeightSpec(f"{prefix}.a1", (rank, h), free=16), WeightSpec(f"{prefix}.a2", (n * d, rank), free=16),
+                    WeightSpec(f"{prefix}.dt_bias", (n * d,), kind="vector")]
+        else:
+            out += [WeightSpec(f"{prefix}.a", (n, h)), WeightSpec(f"{prefix}.dt_bias", (n,), kind="vector")]
+        if p.get("gate_rank") is not None:
+            rank = int(p["gate_rank"])
+            out += [WeightSpec(f"{prefix}.g1", (rank, h), free=16), WeightSpec(f"{prefix}.g2", (n * dv, rank), free=16)]
+        else:
+            out.append(WeightSpec(f"{prefix}.g", (n * dv, h)))
+        return out + [WeightSpec(f"{prefix}.o", (h, n * dv))]
 
     def cache_spec(self):
         return StateSpec((self.heads * self.d * self.dv + (self.taps - 1) * self.channels,), "float32")
@@ -219,10 +243,28 @@ class GatedDelta(Mixer):
         if self.d > rt.kernels.delta_max_dim():
             raise ValueError(f"a state of {self.d} rows a head is not supported: the delta rule kernel takes up to "
                              f"{rt.kernels.delta_max_dim()}")
-        tensors = [weights.get(f"{self.prefix}.{n}") for n in ("q", "k", "v", "b", "a", "g")]
+        # one product, stored in float32, for what the 32-bit passes read: q | k | v | b, then a (a decay a head),
+        # then g (a gate without a bottleneck); a second one, in the compute dtype, for the bottlenecks a1 | g1,
+        # which the products with a2 and g2 read
+        names = ["q", "k", "v", "b"] + ([] if self.decay == "channel" else ["a"]) + (["g"] if self.gate_rank is None else [])
+        tensors = [weights.get(f"{self.prefix}.{n}") for n in names]
         if len({t.dtype for t in tensors}) > 1:
             tensors = [t.to(torch.float32) for t in tensors]
         self.w_in = rt.matrix(torch.cat(tensors, dim=0))
+        low = [weights.get(f"{self.prefix}.{n}") for n in (["a1"] if self.decay == "channel" else []) +
+               (["g1"] if self.gate_rank is not None else [])]
+        if len({t.dtype for t in low}) > 1:
+            low = [t.to(torch.float32) for t in low]
+        self.decay_rank = low[0].shape[0] if self.decay == "channel" else 0
+        # (zero rows behind a1, so that the gate's part of the product's rows starts on a 16-byte boundary)
+        self.low_gate_at = -(-self.decay_rank // 8) * 8
+        if self.decay == "channel" and len(low) > 1 and self.low_gate_at > self.decay_rank:
+            low.insert(1, low[0].new_zeros((self.low_gate_at - self.decay_rank, low[0].shape[1])))
+        self.w_low = rt.matrix(torch.cat(low, dim=0)) if low else None
+        if self.decay == "channel":
+            self.w_a2 = rt.matrix(weights.get(f"{self.prefix}.a2"))
+        if self.gate_rank is not None:
+            self.w_g2 = rt.matrix(weights.get(f"{self.prefix}.g2"))
         self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
         self.conv = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.conv").to(torch.float32) for n in "qkv"], dim=0))
         self.a_log = rt.vector(weights.get(f"{self.prefix}.A_log"))
@@ -236,9 +278,23 @@ class GatedDelta(Mixer):
         raw = ctx.buf("delta.in_f32", (t, self.w_in.shape[0]), torch.float32)
         k.gemm(x, self.w_in, raw, STORE_F32)
         o = ctx.buf("delta.o_f32", (t, n * dv), torch.float32)
-        scratch = ctx.buf("delta.scratch", (k.delta_scratch_floats(t, g, n, d, dv),), torch.float32)
+        channel = self.decay == "channel"
+        scratch = ctx.buf("delta.scratch", (k.delta_scratch_floats(t, g, n, d, dv, channel),), torch.float32)
+        decay_logits = None
+        if self.w_low is not None:
+            from ..ops import STORE
+
+            low = ctx.buf("delta.low", (t, self.w_low.shape[0]), rt.dtype)
+            k.gemm(x, self.w_low, low, STORE)
+        if channel:
+            decay_logits = ctx.buf("delta.decay_f32", (t, n * d), torch.float32)
+            k.gemm(low[:, :self.decay_rank], self.w_a2, decay_logits, STORE_F32)
+        gate = raw[:, self.channels + (1 if channel else 2) * n:]
+        if self.gate_rank is not None:
+            gate = ctx.buf("delta.gate_f32", (t, n * dv), torch.float32)
+            k.gemm(low[:, self.low_gate_at:], self.w_g2, gate, STORE_F32)
         k.delta_rule(raw, g, n, d, dv, self.conv, self.a_log, self.dt_bias, self.unit_eps, ctx.tok_seq, ctx.tok_pos,
-                     ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), scratch, o)
+                     ctx.seqs, ctx.n_seqs, ctx.cache.unit_state(run.cache), scratch, o, channel_decay=decay_logits)
         gated = ctx.buf("delta.normed", (t, n * dv), rt.dtype)
-        k.head_norm_gate(o, n, dv, self.norm, raw[:, self.channels + 2 * n:], self.eps, gated)
+        k.head_norm_gate(o, n, dv, self.norm, gate, self.eps, gated, gate_act=self.gate_act)
         return project_out(ctx, gated, self.w_o, out, accumulate, defer, "delta.out_slices")

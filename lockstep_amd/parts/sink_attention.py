@@ -6,6 +6,7 @@ query head h reads kv head ``h // (H/G)``), at true positions i (query) and j (k
 
     s_h[i, j] = scale * <q_h[i], k_kv(h)[j]> + rel[bucket(i - j), h]            (the bias is optional)
     j is visible to i  iff  lo(i) <= j <= i, where lo(i) is 0, i - window + 1, or the start of i's chunk
+                            (with a window, also if j < keep_first: the first tokens stay visible)
     p_h[i, j] = exp(s_h[i, j]) / (exp(sink_h) + sum_j' exp(s_h[i, j']))         (sink: none, zero, or learned)
     o_h[i]    = sigmoid(g_h[i]) * sum_j p_h[i, j] v_kv(h)[j]                    (the gate is optional)
 
@@ -61,9 +62,10 @@ def distance_buckets(rows: int, farthest: float) -> list[int]:
 class SinkAttention(Mixer):
     """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim`` (queries and keys),
     ``value_dim``, ``position`` (a position-encoding ``PartSpec``), ``scale``, ``window`` / ``chunk``
-    (None or a size; at most one of them), ``sink`` (None, ``"zero"`` or ``"learned"``), ``gate``,
+    (None or a size; at most one of them), ``keep_first`` (with a window: the first that many tokens stay visible), ``sink`` (None, ``"zero"`` or ``"learned"``), ``gate``,
     ``bias`` (biases of q, k, v), ``out_bias``, ``qk_norm`` (None or the eps of a norm over the whole
-    projection), ``head_norm`` (None or the eps of a norm without weights over every head of q and of k), ``shared_kv`` (the values are the keys as projected), ``distance_bias`` (None or
+    projection), ``head_norm`` (None or the eps of a norm over every head of q and of k; without weights, or with ``head_norm_weights`` times
+    ``q.norm`` / ``k.norm`` of ``head_dim`` elements that all heads share), ``shared_kv`` (the values are the keys as projected), ``distance_bias`` (None or
     ``{"farthest": D, "rows": B}``; ``rows`` only sizes random weights, a checkpoint's table says it itself).
     Tensors below the prefix: ``q``, ``k``, ``v``, ``o``; ``g`` (gate); ``q.b``, ``k.b``, ``v.b``;
     ``o.b``; ``q.norm``, ``k.norm``; ``rel [B, H]``; ``sink [H]``."""
@@ -80,6 +82,7 @@ class SinkAttention(Mixer):
         self.scale = float(p["scale"])
         self.window = int(p.get("window") or 0)
         self.chunk = int(p.get("chunk") or 0)
+        self.keep_first = int(p.get("keep_first") or 0)
         self.sink_kind = p.get("sink")
         self.gate = bool(p.get("gate"))
         self.bias = bool(p.get("bias"))
@@ -88,6 +91,11 @@ class SinkAttention(Mixer):
         self.head_norm = None if p.get("head_norm") is None else float(p["head_norm"])
         if self.qk_norm is not None and self.head_norm is not None:
             raise ValueError("a norm over the whole projection and a norm over every head: at most one")
+        self.head_norm_weights = bool(p.get("head_norm_weights"))
+        if self.head_norm_weights and self.head_norm is None:
+            raise ValueError("head_norm_weights belong to a head_norm")
+        if self.keep_first < 0 or (self.keep_first and not self.window):
+            raise ValueError(f"keep_first {self.keep_first} must not be negative and needs a window")
         self.shared_kv = bool(p.get("shared_kv"))
         self.distance_bias = p.get("distance_bias")
         if self.nq % self.nkv:
@@ -129,6 +137,9 @@ class SinkAttention(Mixer):
         if p.get("qk_norm") is not None:
             out += [WeightSpec(f"{prefix}.q.norm", (nq * d,), kind="vector", init="norm"),
                     WeightSpec(f"{prefix}.k.norm", (nkv * d,), kind="vector", init="norm")]
+        if p.get("head_norm") is not None and p.get("head_norm_weights"):
+            out += [WeightSpec(f"{prefix}.q.norm", (d,), kind="vector", init="norm"),
+                    WeightSpec(f"{prefix}.k.norm", (d,), kind="vector", init="norm")]
         if p.get("distance_bias") is not None:
             out.append(WeightSpec(f"{prefix}.rel", (-1, nq), kind="vector", free=int(p["distance_bias"].get("rows") or 32)))
         if p.get("sink") == "learned":
@@ -136,7 +147,8 @@ class SinkAttention(Mixer):
         return out
 
     def cache_spec(self):
-        return PagedKVSpec(self.nkv, self.dk, self.window or None, value_dim=self.dv, chunk=self.chunk or None)
+        return PagedKVSpec(self.nkv, self.dk, self.window or None, value_dim=self.dv, chunk=self.chunk or None,
+                           keep_first=self.keep_first)
 
     def load(self, weights, rt) -> None:
         names = ["q", "k"] + ([] if self.shared_kv else ["v"]) + (["g"] if self.gate else [])
@@ -150,7 +162,7 @@ class SinkAttention(Mixer):
             self.b_in = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.b").to(torch.float32) for n in biased]))
         if self.out_bias:
             self.b_o = rt.vector(weights.get(f"{self.prefix}.o.b"))
-        if self.qk_norm is not None:
+        if self.qk_norm is not None or self.head_norm_weights:
             self.q_norm = rt.vector(weights.get(f"{self.prefix}.q.norm"))
             self.k_norm = rt.vector(weights.get(f"{self.prefix}.k.norm"))
         if self.sink_kind == "learned":
@@ -176,7 +188,7 @@ class SinkAttention(Mixer):
             lo = max(lo, position - self.window + 1)
         if self.chunk:
             lo = max(lo, position // self.chunk * self.chunk)
-        return position - lo + 1
+        return position - lo + 1 + min(self.keep_first, lo)
 
     def mixing_flops(self, tokens: int, start: int) -> float:
         pairs = sum(self._seen(start + i) for i in range(tokens))
@@ -184,11 +196,12 @@ class SinkAttention(Mixer):
 
     def prepare_group(self):
         share = getattr(self.position, "share_key", None)
-        return None if share is None else ("sink_attention", self.window, self.chunk, self.nq, self.nkv, self.dk, self.dv, share())
+        return None if share is None else ("sink_attention", self.window, self.chunk, self.keep_first, self.nq, self.nkv,
+                                           self.dk, self.dv, share())
 
     def _block_key(self):
         # (the blocks of rows and the tiles of keys depend on the heads and the sizes as well)
-        return ("sink_attention", "work", self.window, self.chunk, self.nq, self.nkv, self.dk, self.dv)
+        return ("sink_attention", "work", self.window, self.chunk, self.keep_first, self.nq, self.nkv, self.dk, self.dv)
 
     def _first_seen(self, positions):
         lo = np.zeros_like(positions)
@@ -213,7 +226,7 @@ class SinkAttention(Mixer):
             # two above the longest context only)
             longest = int(ctx.kv_len.max()) + ctx.horizon
             if self.window:
-                longest = min(longest, self.window)
+                longest = min(longest, self.window + self.keep_first)
             if self.chunk:
                 longest = min(longest, self.chunk)
             tiles = 1 << max(0, (-(-longest // TILE_KEYS) - 1).bit_length())
@@ -246,7 +259,8 @@ class SinkAttention(Mixer):
             first = ctx.q_start[seq] + block * block_rows                          # position of a block's first row
             rows = np.minimum(block_rows, ctx.q_len[seq] - block * block_rows)
             last = first + rows - 1
-            tiles = last // tile_keys - self._first_seen(first) // tile_keys + 1    # (as the kernel counts them)
+            lo_tile = self._first_seen(first) // tile_keys
+            tiles = last // tile_keys - lo_tile + 1 + np.minimum(-(-self.keep_first // tile_keys), lo_tile)    # (as the kernel counts them)
             # runs of at least TILES_A_RUN tiles of 32 keys, longer where the step has more work than a few items a CU
             a_run = max(TILES_A_RUN * TILE_KEYS // tile_keys, -(-int(tiles.sum()) * groups // (4 * cus)))
             runs = np.minimum(MAX_RUNS, np.maximum(1, tiles // a_run))
@@ -277,7 +291,8 @@ class SinkAttention(Mixer):
         k.qkv_post(raw, t, nq, nkv, d, dv, self.b_in, self.q_norm, self.k_norm, self.qk_norm or self.head_norm or 0.0, self.position.cos,
                    self.position.sin, self.position.rotary_dim, self.neighbours, ctx.max_position, ctx.tok_seq,
                    ctx.tok_pos, ctx.seqs, group.table, q, key_pages, value_pages, group.page_size,
-                   keys_are_values=self.shared_kv, key_pad=self.dk, per_head=self.head_norm is not None)
+                   keys_are_values=self.shared_kv, key_pad=self.dk, per_head=self.head_norm is not None,
+                   head_weights=self.head_norm_weights)
         key = self._block_key()
         attn = ctx.buf("sink.out", (t, nq * dv), rt.dtype)
         n_items, n_folds, row_tiles = ctx.notes[key]
@@ -287,7 +302,8 @@ class SinkAttention(Mixer):
         gate = raw[:, raw.shape[1] - nq * dv:] if self.gate else None
         k.sink_attention(q, nq, nkv, self.dk, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                          work[:4 * n_items], n_items, row_tiles, self.scale, self.window, self.chunk, self.sink,
-                         self.by_distance, gate, attn, work[4 * n_items:] if n_folds else None, n_folds, part)
+                         self.by_distance, gate, attn, work[4 * n_items:] if n_folds else None, n_folds, part,
+                         keep_first=self.keep_first)
         if self.b_o is not None:
             # (a product with an output bias is added to the stream at once, then the bias: the same order
             # of additions at every batch size)

@@ -17,6 +17,17 @@ v_first`` of the same token before they are cached, with its scalar ``lambda``.
 The projections are one matrix product over ``[Wq; Wk; Wv]`` stored in float32; one pass adds the
 biases, rotates, mixes values and writes queries, keys and values; one launch runs the attention
 of all requests of the step.
+
+With ``mix = "weights"`` the heads exchange their weights after each head's own softmax instead:
+
+    p_g[i, j]   = exp(raw_g[i, j]) / (exp(sink_g) + sum_j' exp(raw_g[i, j']))   (visible j'; the sink is optional)
+    o_h[i]      = sigmoid(gate_h[i]) * sum_j (sum_g talk[h, g] p_g[i, j]) v_kv(h)[j]    (the gate is optional)
+
+A head's mixed weights are applied to the values of its own key/value head.  The sink has no key and no
+value and is not mixed.  This form may also have ``shared_kv`` (no value projection: the values are the
+keys as projected, before rotation) and rotates neighbouring pairs where the position encoding says so;
+its pass in front of the attention is the one that the attention with a sink uses.  The keys are walked
+twice (statistics, then weights), because a mixed weight needs every head's finished sum.
 """
 
 from __future__ import annotations
@@ -41,7 +52,10 @@ class TalkingAttention(Mixer):
     ``value_dim``, ``position`` (a position-encoding ``PartSpec``), ``window``, ``keep_first``,
     ``scale``, ``bias`` (biases of q, k, v), ``v_mix`` (None, ``"source"`` or ``"mix"``).  Tensors below
     the prefix: ``q``, ``k``, ``v``, ``o``, ``talk`` ``[H, H]``, with ``bias`` also ``q.b``, ``k.b``,
-    ``v.b``, with ``v_mix`` also the scalar ``vmix`` (unused by the source layer)."""
+    ``v.b``, with ``v_mix`` also the scalar ``vmix`` (unused by the source layer).
+    ``mix`` (``"scores"``, the default, or ``"weights"``); with ``"weights"`` also ``sink`` (None, ``"zero"``
+    or ``"learned"``: the tensor ``sink [H]``), ``gate`` (the tensor ``g [H*vdim, hidden]``) and ``shared_kv``
+    (no tensor ``v``), and no ``v_mix``."""
 
     graph_safe = True
 
@@ -61,10 +75,27 @@ class TalkingAttention(Mixer):
             raise ValueError(f"window {self.window} must be positive and keep_first {self.keep_first} not negative")
         if self.v_mix not in (None, "source", "mix"):
             raise ValueError(f"v_mix must be None, 'source' or 'mix', got {self.v_mix!r}")
+        self.mix = p.get("mix") or "scores"
+        self.sink_kind, self.gate, self.shared_kv = p.get("sink"), bool(p.get("gate")), bool(p.get("shared_kv"))
+        if self.mix not in ("scores", "weights"):
+            raise ValueError(f"mix must be 'scores' or 'weights', got {self.mix!r}")
+        if self.sink_kind not in (None, "zero", "learned"):
+            raise ValueError(f"sink must be None, 'zero' or 'learned', got {self.sink_kind!r}")
+        if self.mix == "scores" and (self.sink_kind or self.gate or self.shared_kv):
+            raise ValueError("a sink, a gate and keys as values come with mix = 'weights'")
+        if self.mix == "weights" and self.v_mix is not None:
+            raise ValueError("values are mixed across layers with mix = 'scores' only")
+        if self.shared_kv and self.d != self.dv:
+            raise ValueError(f"keys of {self.d} elements cannot be the values of {self.dv}")
+        # (the pass in front of mixed weights pads a head of the queries and the cached keys to 16 bytes' worth)
+        self.dk = -(-self.d // 8) * 8 if self.mix == "weights" else self.d
         self.position = build_part(p["position"], prefix)
         if self.position.rotary_dim > self.d:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head size {self.d}")
-        self.w_qkv = self.w_o = self.b_qkv = self.talk = self.vmix = None
+        self.neighbours = bool(getattr(self.position, "neighbours", False))
+        if self.neighbours and self.mix == "scores":
+            raise ValueError("mix = 'scores' rotates the halves of a head; neighbouring pairs come with mix = 'weights'")
+        self.w_qkv = self.w_o = self.b_qkv = self.talk = self.vmix = self.sink = None
 
     def parts(self):
         return (self.position,)
@@ -75,31 +106,44 @@ class TalkingAttention(Mixer):
         h, nq, nkv = int(p["hidden_size"]), int(p["num_heads"]), int(p["num_kv_heads"])
         d, dv = int(p["head_dim"]), int(p["value_dim"])
         out = [WeightSpec(f"{prefix}.q", (nq * d, h)), WeightSpec(f"{prefix}.k", (nkv * d, h)),
-               WeightSpec(f"{prefix}.v", (nkv * dv, h)), WeightSpec(f"{prefix}.o", (h, nq * dv)),
+               WeightSpec(f"{prefix}.o", (h, nq * dv)),
                WeightSpec(f"{prefix}.talk", (nq, nq), kind="vector", init="identity")]
+        if not p.get("shared_kv"):
+            out.append(WeightSpec(f"{prefix}.v", (nkv * dv, h)))
+        if p.get("gate"):
+            out.append(WeightSpec(f"{prefix}.g", (nq * dv, h)))
+        if p.get("sink") == "learned":
+            out.append(WeightSpec(f"{prefix}.sink", (nq,), kind="vector"))
         if p.get("bias"):
-            out += [WeightSpec(f"{prefix}.q.b", (nq * d,), kind="vector"), WeightSpec(f"{prefix}.k.b", (nkv * d,), kind="vector"),
-                    WeightSpec(f"{prefix}.v.b", (nkv * dv,), kind="vector")]
+            out += [WeightSpec(f"{prefix}.q.b", (nq * d,), kind="vector"), WeightSpec(f"{prefix}.k.b", (nkv * d,), kind="vector")]
+            if not p.get("shared_kv"):
+                out.append(WeightSpec(f"{prefix}.v.b", (nkv * dv,), kind="vector"))
         if p.get("v_mix"):
             out.append(WeightSpec(f"{prefix}.vmix", (), kind="vector", init="unit"))
         return out
 
     def cache_spec(self):
-        return PagedKVSpec(self.nkv, self.d, self.window, value_dim=self.dv, keep_first=self.keep_first)
+        return PagedKVSpec(self.nkv, self.dk, self.window, value_dim=self.dv, keep_first=self.keep_first)
 
     def load(self, weights, rt) -> None:
-        q, k, v = (weights.get(f"{self.prefix}.{n}") for n in "qkv")
-        if len({q.dtype, k.dtype, v.dtype}) > 1:
-            q, k, v = q.to(torch.float32), k.to(torch.float32), v.to(torch.float32)
-        self.w_qkv = rt.matrix(torch.cat([q, k, v], dim=0))
+        names = ["q", "k"] + ([] if self.shared_kv else ["v"]) + (["g"] if self.gate else [])
+        mats = [weights.get(f"{self.prefix}.{n}") for n in names]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.to(torch.float32) for m in mats]
+        self.w_qkv = rt.matrix(torch.cat(mats, dim=0))
         self.w_o = rt.matrix(weights.get(f"{self.prefix}.o"))
         self.talk = rt.vector(weights.get(f"{self.prefix}.talk"))
         if self.bias:
-            self.b_qkv = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.b").to(torch.float32) for n in "qkv"]))
+            biased = ["q", "k"] + ([] if self.shared_kv else ["v"])
+            self.b_qkv = rt.vector(torch.cat([weights.get(f"{self.prefix}.{n}.b").to(torch.float32) for n in biased]))
         if self.v_mix == "mix":
             self.vmix = rt.vector(weights.get(f"{self.prefix}.vmix").reshape(1))
+        if self.sink_kind == "learned":
+            self.sink = rt.vector(weights.get(f"{self.prefix}.sink"))
+        elif self.sink_kind == "zero":
+            self.sink = rt.vector(torch.zeros(self.nq, dtype=torch.float32))
         rt.kernels.mixers_lib()
-        rt.kernels.talking_lib(self.nq, self.nkv, self.d, self.dv)
+        rt.kernels.talking_lib(self.nq, self.nkv, self.dk, self.dv)
         if hasattr(self.position, "bind"):
             self.position.bind(rt)
 
@@ -107,7 +151,8 @@ class TalkingAttention(Mixer):
         """Scores, their mixing over the heads and value products over the (query, key) pairs a query sees."""
         pairs = sum(min(start + i + 1, self.window + min(self.keep_first, max(0, start + i + 1 - self.window)))
                     for i in range(tokens))
-        return (2.0 * self.d + 2.0 * self.dv + 2.0 * self.nq) * self.nq * pairs
+        # (mixed weights walk the keys twice: the scores are formed once more)
+        return ((4.0 if self.mix == "weights" else 2.0) * self.d + 2.0 * self.dv + 2.0 * self.nq) * self.nq * pairs
 
     def prepare_group(self):
         share = getattr(self.position, "share_key", None)
@@ -172,6 +217,8 @@ class TalkingAttention(Mixer):
         group, key_pages, value_pages = ctx.cache.unit_pages(run.cache)
         if not run.writes_cache:
             raise ValueError("a talking-heads attention layer writes its own keys and values")
+        if self.mix == "weights":
+            return self._forward_mixed_weights(ctx, run, x, out, accumulate, defer)
         raw = ctx.buf("talking.qkv_f32", (t, nq * d + nkv * (d + dv)), torch.float32)
         k.gemm(x, self.w_qkv, raw, STORE_F32)
         q = ctx.buf("talking.q", (t, nq * d), rt.dtype)
@@ -190,4 +237,32 @@ class TalkingAttention(Mixer):
         k.talk_attention(q, nq, nkv, d, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
                          work[:4 * n_items], n_items, self.talk, self.scale, self.window, self.keep_first, attn,
                          work[4 * n_items:] if n_folds else None, n_folds, part, part_rows)
+        return project_out(ctx, attn, self.w_o, out, accumulate, defer, "talking.out_slices")
+
+    def _forward_mixed_weights(self, ctx, run, x, out, accumulate: bool, defer: bool):
+        """``mix = "weights"``: the projection (with the gate's logits behind it), the pass that rotates and writes the
+        cache, the two passes of the attention, the output projection."""
+        rt = ctx.rt
+        k = rt.kernels
+        t = ctx.n_tokens
+        nq, nkv, d, dv = self.nq, self.nkv, self.d, self.dv
+        group, key_pages, value_pages = ctx.cache.unit_pages(run.cache)
+        raw = ctx.buf("talking.in_f32", (t, self.w_qkv.shape[0]), torch.float32)
+        k.gemm(x, self.w_qkv, raw, STORE_F32)
+        q = ctx.buf("talking.q", (t, nq * self.dk), rt.dtype)
+        k.qkv_post(raw, t, nq, nkv, d, dv, self.b_qkv, None, None, 0.0, self.position.cos, self.position.sin,
+                   self.position.rotary_dim, self.neighbours, ctx.max_position, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
+                   group.table, q, key_pages, value_pages, group.page_size, keys_are_values=self.shared_kv,
+                   key_pad=self.dk)
+        key = self._block_key()
+        attn = ctx.buf("talking.out", (t, nq * dv), rt.dtype)
+        n_items, n_folds, part_rows = ctx.notes[key]
+        work = ctx.block(key)
+        part = ctx.buf("talking.part", (n_items * part_rows * nq * (dv + 2),), torch.float32) if n_folds else None
+        stats = ctx.buf("talking.stats", (n_items * 16 * nq * 2,), torch.float32)
+        gate = raw[:, raw.shape[1] - nq * dv:] if self.gate else None
+        k.talk_attention(q, nq, nkv, self.dk, dv, key_pages, value_pages, group.page_size, group.table, ctx.seqs,
+                         work[:4 * n_items], n_items, self.talk, self.scale, self.window, self.keep_first, attn,
+                         work[4 * n_items:] if n_folds else None, n_folds, part, part_rows, mix_weights=True,
+                         sink=self.sink, stats=stats, gate=gate)
         return project_out(ctx, attn, self.w_o, out, accumulate, defer, "talking.out_slices")
