@@ -38,7 +38,10 @@ measures the Bikovik design (talking-heads attention over a window that keeps th
 HGRN2 and retention layers, Dynamic Tanh norms, a clamped gated feed-forward) and the Biberax
 design (chunked and biased attention with a sink and an output gate, routed experts) or, with
 ``--designs qwen3,toripel``, the Toripel design (a residual stream of four copies, the gated delta rule, windowed
-attention, attention over a cached latent, experts named by a table; ``--designs``
+attention, attention over a cached latent, experts named by a table) or, with ``--designs qwen3,toripel,narurax``,
+the Narurax design (an embedding that adds a table of token pairs, mixer inputs shifted towards the token before, the
+delta rule with a decay a channel, attention whose weights are mixed over the heads, attention with a norm a head,
+windows that keep the first tokens, experts with sigmoid scores on their input; ``--designs``
 chooses) beside the Qwen3 decoder at the same layer sizes (width, feed-forward, heads, head size, layers, vocabulary), both
 with random weights: prefill of one prompt and decode steps at batch 1 and 8, each with its
 fraction of the roofline.
@@ -421,6 +424,30 @@ def toripel_like(qwen, layers: int, window: int = 4096, experts: int = 32, top: 
                              "embedding": {"scale": 1.0}, "norm": {"eps": qwen.rms_norm_eps}, "streams": streams, "layers": out})
 
 
+def narurax_like(qwen, layers: int, window: int = 4096, keep_first: int = 4, experts: int = 32, top: int = 4):
+    """A Narurax configuration at the layer sizes of the Qwen3 configuration ``qwen``: the layers cycle through the
+    delta rule with a decay a channel, attention whose weights are mixed over the heads, and twice attention with a
+    norm a head and a one in the denominator; every mixer has the heads and head size of the Qwen3 attention, the
+    windows keep the first tokens.  A token's feed-forward multiplies with as many weights as the dense one: ``top``
+    experts of ``1 / top`` of the dense size each, chosen by sigmoid scores that multiply the experts' input."""
+    from lockstep_amd.config import config_from_dict
+
+    heads, kv, d = qwen.num_attention_heads, qwen.num_key_value_heads, qwen.head_dim
+    moe = {"kind": "moe", "expert": {"ff": qwen.intermediate_size // top}, "router": {"experts": experts, "top": top}}
+    mask = {"size": window, "keep_first": keep_first}
+    delta = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4}
+    mixing = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": mask,
+              "rot": {"dims": d, "base": qwen.rope_theta}}
+    normed = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": mask,
+              "rot": {"dims": d, "base": qwen.rope_theta, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    cycle = [{"type": "channel_delta", "mixer": delta, "mlp": moe}, {"type": "attention", "mixer": mixing, "mlp": moe},
+             {"type": "attention_2", "mixer": normed, "mlp": moe}, {"type": "attention_2", "mixer": normed, "mlp": moe}]
+    return config_from_dict({"architecture": "Narurax", "vocab": qwen.vocab_size, "width": qwen.hidden_size,
+                             "norm": {"eps": qwen.rms_norm_eps},
+                             "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+                             "layers": [cycle[i % 4] for i in range(layers)]})
+
+
 def designs_record(args) -> dict:
     """Prefill and decode of the other designs beside Qwen3 at equal layer sizes."""
     import gc
@@ -439,13 +466,18 @@ def designs_record(args) -> dict:
            "prefill_tokens": args.prefill_len, "prompt_len": args.prompt_len, "steps": args.steps,
            "data": "synthetic: uniform random token ids, random weights", "designs": {}}
     makers = {"qwen3": lambda: qwen, "bikovik": lambda: bikovik_like(qwen, layers), "biberax": lambda: biberax_like(qwen, layers),
-              "toripel": lambda: toripel_like(qwen, layers)}
+              "toripel": lambda: toripel_like(qwen, layers), "narurax": lambda: narurax_like(qwen, layers)}
     for name in args.designs.split(","):
         if name not in makers:
             raise SystemExit(f"--designs: {name!r} is not one of {', '.join(makers)}")
         config = makers[name]()
         print(f"[bench] drawing random weights for {name} at {args.model} sizes", file=sys.stderr, flush=True)
         tensors = random_tensors(config, seed=0, std=0.02, norm_std=0.0, dtype=torch.bfloat16)
+        if name == "narurax":          # bottlenecks of half a head's size (the random-weights mode draws narrow ones)
+            rank = max(16, qwen.head_dim // 2)
+            for key in [k for k in tensors if k.endswith((".mix.a1", ".mix.g1", ".mix.a2", ".mix.g2"))]:
+                shape = (rank, tensors[key].shape[1]) if key.endswith("1") else (tensors[key].shape[0], rank)
+                tensors[key] = (torch.randn(shape) * 0.02).to(torch.bfloat16)
         model = model_from_tensors(config, tensors, dtype=dtype)
         del tensors
         work = Workload(model)
@@ -614,7 +646,7 @@ def main(argv=None) -> int:
                         "scheduler; contexts: prefill and decode at the context lengths of --contexts; designs: "
                         "the Bikovik and Biberax designs beside Qwen3 at the layer sizes of --model")
     p.add_argument("--contexts", default="4096,8192,16384", help="contexts: the context lengths, comma separated")
-    p.add_argument("--designs", default="qwen3,bikovik,biberax", help="designs: which of qwen3, bikovik, biberax, toripel, comma separated")
+    p.add_argument("--designs", default="qwen3,bikovik,biberax", help="designs: which of qwen3, bikovik, biberax, toripel, narurax, comma separated")
     p.add_argument("--repeats", type=int, default=5, help="timed runs; the median is reported with the spread")
     p.add_argument("--requests", type=int, default=0, help="serve: only the first N requests of the workload")
     p.add_argument("--prefill-chunk", type=int, default=None, help="serve: prompt portion (0: whole prompts)")

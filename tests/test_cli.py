@@ -101,3 +101,21 @@ def test_init_writes_a_toripel_folder_from_its_preset(tmp_path):
         assert name in names, name
     assert "l3.mix.dkv" not in names and "l3.mlp.table" not in names and "l0.mlp.router" not in names
     assert tuple(handle.shape("l0.mlp.table")) == (640, 2) and tuple(handle.shape("l2.mix.dkv")) == (48, 128)
+
+
+def test_init_writes_a_narurax_folder_from_its_preset(tmp_path):
+    from lockstep_amd.config import NaruraxConfig, config_from_dir
+    from lockstep_amd.weights import SafetensorsFile
+
+    done = run("init", "--preset", "narurax-tiny", "--out", str(tmp_path / "k"), "--seed", "2")
+    assert done.returncode == 0, done.stderr
+    config = config_from_dir(tmp_path / "k")
+    assert isinstance(config, NaruraxConfig) and config.width == 128 and len(config.layers) == 4
+    handle = SafetensorsFile(tmp_path / "k" / "model.safetensors")
+    names = handle.keys()
+    for name in ("embed", "bigram", "head", "final.norm", "l0.shift", "l3.shift", "l0.mix.q.conv", "l0.mix.A_log", "l0.mix.a1",
+                 "l0.mix.g2", "l0.mlp.router", "l0.mlp.e7.down", "l1.mix.talk", "l1.mix.sink", "l1.mix.g", "l2.mix.q.norm",
+                 "l2.mix.k.b", "l2.mix.o.b"):
+        assert name in names, name
+    assert "l1.mix.v" not in names and "l3.mlp.router" not in names and "l0.mlp.router.b" not in names and "l0.mix.a" not in names
+    assert tuple(handle.shape("bigram")) == (510, 128) and tuple(handle.shape("l0.mix.dt_bias")) == (128,)

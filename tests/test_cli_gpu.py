@@ -118,3 +118,21 @@ def test_a_toripel_folder_generates_what_the_plain_model_generates(tmp_path):
     cut = run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", "--prefill-chunk", "9",
               "--max-batched-tokens", "20", "--block-size", "8", "--num-blocks", "40", "--decode-burst", "1", *args)
     assert cut == want
+
+
+def test_a_narurax_folder_generates_what_the_plain_model_generates(tmp_path):
+    from lockstep_amd.weights.safetensors_io import open_model_tensors
+    from plain.narurax_plain import PlainNarurax
+
+    folder = tmp_path / "k"
+    subprocess.run([*LOCKSTEP, "init", "--preset", "narurax-tiny", "--out", str(folder), "--seed", "3", "--std", "0.2"],
+                   check=True, capture_output=True, timeout=300)
+    tensors = {name: handle.get(key) for name, (handle, key) in open_model_tensors(folder).items()}
+    plain = PlainNarurax(json.loads((folder / "config.json").read_text()), tensors)
+    prompts = [random_tokens(n, 640, seed=90 + n) for n in (3, 21, 70)]
+    want = {f"r{i:02d}": plain.generate_greedy(p, 6) for i, p in enumerate(prompts)}
+    args = [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))]
+    assert run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", *args) == want
+    cut = run("run", "--model", str(folder), "--dtype", "float32", "--max-new-tokens", "6", "--prefill-chunk", "9",
+              "--max-batched-tokens", "20", "--block-size", "8", "--num-blocks", "40", "--decode-burst", "1", *args)
+    assert cut == want
