@@ -590,6 +590,64 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const float* __restric
   if (first_row) kept[c] = n[(long)(m.q_off + m.q_len - 1) * ldn + c];
 }
 
+// ---------------------------------------------------------------------------
+// A step of single tokens: the residual addition that the last sublayer left, the RMS norm and the token shift in one
+// launch.  h[t] += P[0][t] + P[1][t] + ... (P may be null); n = h[t] / sqrt(mean(h[t]^2) + eps) * weight;
+// out[t] = n + (kept - n) * mu with `kept` the request's state (zeros at its first token), which then becomes n.
+// The additions and the sum of squares follow the order of the norm's own launch (thread t adds the squares of the
+// elements 1024 c + 4 t + {0..3}, c ascending; a butterfly over the wave; the waves in order), so a token's bits do
+// not depend on whether it was decoded alone or stood in a prompt's portion.  width % 4 == 0.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(float* __restrict__ h, const float* __restrict__ P,
+                                                                int slices, int p_rows, const float* __restrict__ weight,
+                                                                const float* __restrict__ mu, const int* __restrict__ tok_seq,
+                                                                const int* __restrict__ tok_pos,
+                                                                const SeqMeta* __restrict__ seqs, float* __restrict__ state,
+                                                                long state_stride, T* __restrict__ out, int width, long ldh,
+                                                                long ld_out, float eps) {
+  __shared__ float wave_part[4];
+  const long row = blockIdx.x;
+  float* hrow = h + row * ldh;
+  float part = 0.f;
+  for (int base = 4 * threadIdx.x; base < width; base += 1024) {
+    f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+    const f32x4 old = *reinterpret_cast<const f32x4*>(hrow + base);
+    for (int s = 0; s < slices; ++s) {
+      const f32x4 p = *reinterpret_cast<const f32x4*>(P + ((long)s * p_rows + row) * width + base);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) total[e] = total[e] + p[e];
+    }
+    f32x4 fresh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) fresh[e] = old[e] + total[e];
+    if (slices > 0) *reinterpret_cast<f32x4*>(hrow + base) = fresh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part = part + fresh[e] * fresh[e];
+  }
+  part = wave_sum(part);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  const float total = ((wave_part[0] + wave_part[1]) + wave_part[2]) + wave_part[3];
+  const float scale = 1.0f / sqrtf(total / (float)width + eps);
+  float* kept = state + (long)seqs[tok_seq[row]].table_row * state_stride;
+  const bool first = tok_pos[row] == 0;
+  T* dst = out + row * ld_out;
+  for (int base = 4 * threadIdx.x; base < width; base += 1024) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(hrow + base);  // this thread wrote it above
+    const f32x4 w = *reinterpret_cast<const f32x4*>(weight + base);
+    const f32x4 m = *reinterpret_cast<const f32x4*>(mu + base);
+    const f32x4 before = *reinterpret_cast<const f32x4*>(kept + base);
+    f32x4 n;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      n[e] = (v[e] * scale) * w[e];
+      dst[base + e] = from_f32<T>(n[e] + ((first ? 0.f : before[e]) - n[e]) * m[e]);
+    }
+    *reinterpret_cast<f32x4*>(kept + base) = n;
+  }
+}
+
 }  // namespace ls
 
 LS_DEFINE_ERROR_API
@@ -656,6 +714,31 @@ extern "C" int ls_token_shift(int out_dtype, const float* n, long ldn, const flo
   else
     return fail("token_shift: unknown dtype %d", out_dtype);
   return check_launch("token_shift");
+}
+
+extern "C" int ls_add_rmsnorm_shift(int out_dtype, float* h, const float* P, int slices, int p_rows, const float* weight,
+                                    const float* mu, const int* tok_seq, const int* tok_pos, const void* seqs, float* state,
+                                    long state_stride, void* out, int n_rows, int width, long ldh, long ld_out, float eps,
+                                    void* stream) {
+  LS_REQUIRE(n_rows > 0 && width > 0 && width % 4 == 0 && ldh >= width && ldh % 4 == 0 && ld_out >= width &&
+                 state_stride >= width && state_stride % 4 == 0 && eps > 0.f,
+             "add_rmsnorm_shift: bad sizes (rows of a multiple of four floats)");
+  LS_REQUIRE(h && weight && mu && tok_seq && tok_pos && seqs && state && out, "add_rmsnorm_shift: null operand");
+  LS_REQUIRE(!P ? slices == 0 : (slices > 0 && p_rows >= n_rows), "add_rmsnorm_shift: bad slice sums");
+  LS_REQUIRE(reinterpret_cast<uintptr_t>(h) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
+                 reinterpret_cast<uintptr_t>(mu) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 &&
+                 (!P || reinterpret_cast<uintptr_t>(P) % 16 == 0),
+             "add_rmsnorm_shift: operands must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (out_dtype == kF32)
+    hipLaunchKernelGGL(add_rmsnorm_shift_kernel<float>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight, mu,
+                       tok_seq, tok_pos, (const SeqMeta*)seqs, state, state_stride, (float*)out, width, ldh, ld_out, eps);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL(add_rmsnorm_shift_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, s, h, P, slices, p_rows, weight, mu,
+                       tok_seq, tok_pos, (const SeqMeta*)seqs, state, state_stride, (bf16_t*)out, width, ldh, ld_out, eps);
+  else
+    return fail("add_rmsnorm_shift: unknown dtype %d", out_dtype);
+  return check_launch("add_rmsnorm_shift");
 }
 
 extern "C" int ls_glu_clamped(int out_dtype, const float* x, long ldx, void* out, long ldo, int rows, int width,

@@ -65,6 +65,11 @@ int ls_embed_pair(int dtype, const int* tokens, const int* tok_seq, const int* t
 
 // out [T][ldo] = n[t] + (n[t-1] - n[t]) * mu, n [T][ldn] float; the row before a portion's first one is the request's
 // state (width floats a slot; zeros at a request's first token), which is left as the portion's last row.
+// A step of single tokens: h[t] += P[0][t] + ... (P null: nothing to add), the RMS norm with `weight`, and the shift
+// with the request's state, which becomes the token's normed row; one launch.  width % 4 == 0.
+int ls_add_rmsnorm_shift(int out_dtype, float* h, const float* P, int slices, int p_rows, const float* weight,
+                         const float* mu, const int* tok_seq, const int* tok_pos, const void* seqs, float* state,
+                         long state_stride, void* out, int n_rows, int width, long ldh, long ld_out, float eps, void* stream);
 int ls_token_shift(int out_dtype, const float* n, long ldn, const float* mu, const int* tok_seq, const int* tok_pos,
                    const void* seqs, float* state, long state_stride, void* out, long ldo, int n_tokens, int width,
                    void* stream);

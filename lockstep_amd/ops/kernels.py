@@ -1423,6 +1423,36 @@ class Kernels:
             c_long(state.stride(0)), _ptr(out), c_int(t), c_int(table.shape[1]), c_long(out.stride(0)), c_float(scale),
             _stream()))
 
+    def add_rmsnorm_shift(self, h: torch.Tensor, partials, weight: torch.Tensor, eps: float, mu: torch.Tensor, tok_seq,
+                          tok_pos, seqs, state: torch.Tensor, out: torch.Tensor) -> None:
+        """For a step of single tokens, in one launch: ``h[t] += partials[0][t] + partials[1][t] + ...`` (``partials``
+        may be None), ``n = rmsnorm(h[t]) * weight`` as ``rmsnorm`` computes it, ``out[t] = n + (kept - n) * mu`` with
+        the request's row of ``state`` (zeros at its first token), which is then left as ``n``."""
+        _rows_ok(h, "add_rmsnorm_shift h"); _rows_ok(out, "add_rmsnorm_shift out")
+        t, width = h.shape
+        if not (h.dtype == torch.float32 and out.dtype in DTYPE_CODE and tuple(out.shape) == (t, width) and width % 4 == 0):
+            raise KernelError("add_rmsnorm_shift works on float32 rows of a multiple of four elements")
+        self._f32_vector(weight, width, "add_rmsnorm_shift weight"); self._f32_vector(mu, width, "add_rmsnorm_shift mu")
+        slices = p_rows = 0
+        if partials is not None:
+            if not (partials.is_cuda and partials.dtype == torch.float32 and partials.is_contiguous() and partials.dim() == 3
+                    and partials.shape[2] == width and partials.shape[1] >= t):
+                raise KernelError("add_rmsnorm_shift partials [slices, rows, width]")
+            slices, p_rows = partials.shape[0], partials.shape[1]
+        if not (state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+                and state.shape[1] >= width):
+            raise KernelError(f"add_rmsnorm_shift state must be float32 [slots, >= {width}]")
+        for name, v in (("tok_seq", tok_seq), ("tok_pos", tok_pos)):
+            if not (v.is_cuda and v.dtype == torch.int32 and v.is_contiguous() and v.numel() >= t):
+                raise KernelError(f"add_rmsnorm_shift {name}: int32, one entry a token")
+        if t == 0:
+            return
+        lib = self.mixers_lib()
+        self._launch(lib, lib.ls_add_rmsnorm_shift, (
+            c_int(DTYPE_CODE[out.dtype]), _ptr(h), _ptr(partials), c_int(slices), c_int(p_rows), _ptr(weight), _ptr(mu),
+            _ptr(tok_seq), _ptr(tok_pos), _ptr(seqs), _ptr(state), c_long(state.stride(0)), _ptr(out), c_int(t), c_int(width),
+            c_long(h.stride(0)), c_long(out.stride(0)), c_float(eps), _stream()))
+
     def token_shift(self, normed: torch.Tensor, mu: torch.Tensor, tok_seq, tok_pos, seqs, state: torch.Tensor,
                     out: torch.Tensor) -> None:
         """``out[t] = n[t] + (n[t-1] - n[t]) * mu`` for the float32 rows ``normed`` of the step, ``n[t-1]`` being the row

@@ -48,6 +48,10 @@ class PreNormResidual(Arrangement):
         if self.shift_name:
             self.width = int(layer_spec.part("mixer_norm")["size"])
             self._fuse_mixer = False          # (the shift stands between the norm and the mixer)
+        # one launch for addition, norm and shift where the norm is a plain RMS norm over rows of whole vectors of four
+        norm = self.mixer_norm
+        self._shift_fused = bool(self.shift_name) and getattr(norm, "kind", "") == "rmsnorm" and norm.copies == 1 \
+            and self._norm1_pending and self.width % 4 == 0
 
     def state_spec(self):
         return StateSpec((self.width,), "float32") if self.shift_name else None
@@ -114,14 +118,20 @@ class PreNormResidual(Arrangement):
             mixed = self._mixer.forward(ctx, run, h, h, accumulate=True, norm=self.mixer_norm)
         else:
             x = ctx.buf("block.normed", (ctx.n_tokens, h.shape[1]), rt.dtype)
-            # (with a token shift the norm's rows stay in float32, and the shift writes what the mixer reads)
-            n = ctx.buf("block.unshifted", (ctx.n_tokens, h.shape[1]), __import__("torch").float32) if self.shift_name else x
-            if pending is not None:
-                self.mixer_norm.forward(ctx, h, n, pending=pending)
+            if self._shift_fused and ctx.single_tokens:
+                # a step of single tokens: the addition that is still open, the norm and the shift in one launch
+                rt.kernels.add_rmsnorm_shift(h, None if pending is None else pending.partials, self.mixer_norm.weight,
+                                             self.mixer_norm.eps, self.shift, ctx.tok_seq, ctx.tok_pos, ctx.seqs,
+                                             ctx.cache.unit_state(run.state), x)
             else:
-                self.mixer_norm.forward(ctx, h, n)
-            if self.shift_name:
-                rt.kernels.token_shift(n, self.shift, ctx.tok_seq, ctx.tok_pos, ctx.seqs, ctx.cache.unit_state(run.state), x)
+                # (with a token shift the norm's rows stay in float32, and the shift writes what the mixer reads)
+                n = ctx.buf("block.unshifted", (ctx.n_tokens, h.shape[1]), __import__("torch").float32) if self.shift_name else x
+                if pending is not None:
+                    self.mixer_norm.forward(ctx, h, n, pending=pending)
+                else:
+                    self.mixer_norm.forward(ctx, h, n)
+                if self.shift_name:
+                    rt.kernels.token_shift(n, self.shift, ctx.tok_seq, ctx.tok_pos, ctx.seqs, ctx.cache.unit_state(run.state), x)
             if self._defer_mixer:
                 mixed = self._mixer.forward(ctx, run, x, h, accumulate=True, defer=True)
             else:
