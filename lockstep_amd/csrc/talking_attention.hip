@@ -81,6 +81,7 @@ __device__ __forceinline__ typename Atom<T>::vec_t load_or_zero(const T* p, bool
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+constexpr int kFoldAtOnce = 16;  // runs whose statistics the second pass requests together (the host deals a row block to at most as many)
 constexpr int kStatRows = 16;   // rows of a work item in `stats` (also for decoded tokens, which use row 0)
 
 // MODE 0: the heads' scores are mixed before the softmax.  MODE 1 / 2: the two passes that mix the heads' weights.
@@ -139,10 +140,22 @@ __global__ __launch_bounds__(64 * NW) void talk_attention_kernel(
       const int h = w * HPW + x;
       const float* st = stats + (((long)(blockIdx.x - run) * kStatRows + (row_ok ? l16 : 0)) * H + h) * 2;
       const long stride = (long)kStatRows * H * 2;
+      // (the statistics of up to kFoldAtOnce runs are requested together: one wait instead of one a run)
+      float mk[kFoldAtOnce], lk[kFoldAtOnce];
+#pragma unroll
+      for (int k = 0; k < kFoldAtOnce; ++k) {
+        const long at = (long)min(k, n_runs - 1) * stride;
+        mk[k] = st[at];
+        lk[k] = st[at + 1];
+      }
       float top = sink ? sink[h] : kNegSentinel;
-      for (int k = 0; k < n_runs; ++k) top = fmaxf(top, st[k * stride]);
+#pragma unroll
+      for (int k = 0; k < kFoldAtOnce; ++k) top = fmaxf(top, k < n_runs ? mk[k] : kNegSentinel);
+      for (int k = kFoldAtOnce; k < n_runs; ++k) top = fmaxf(top, st[k * stride]);
       float total = 0.f;
-      for (int k = 0; k < n_runs; ++k) total = total + st[k * stride + 1] * softmax_exp<T>(st[k * stride] - top);
+#pragma unroll
+      for (int k = 0; k < kFoldAtOnce; ++k) total = total + (k < n_runs ? lk[k] * softmax_exp<T>(mk[k] - top) : 0.f);
+      for (int k = kFoldAtOnce; k < n_runs; ++k) total = total + st[k * stride + 1] * softmax_exp<T>(st[k * stride] - top);
       if (sink) total = total + softmax_exp<T>(sink[h] - top);
       m_all[x] = top;
       inv_all[x] = row_ok && total > 0.f ? 1.0f / total : 0.f;

@@ -272,6 +272,33 @@ def test_a_long_prompt_and_decoding_after_it(models, dtype):
         cache.close("r")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_windows_whose_keys_are_dealt_to_runs(tmp_path, dtype):
+    """Windows of hundreds of keys with kept first tokens that fill more than a tile: the late row blocks of a prompt
+    of 900 tokens and every decoded token deal their tiles (the kept ones first) to several work items, whose
+    statistics and outputs are folded; the mixed weights need every run's statistics before any run's output."""
+    from lockstep_amd import load_model
+
+    raw = config(64, 96, [bare(mixing(4, 2, 24, window=700, keep_first=37, scale=0.5, dims=16)),
+                          bare(normed(4, 2, 16, 40, window=600, keep_first=70, scale=0.5, scaling=(4.0, 1.0, 8.0, 32)))])
+    tensors = make_tensors(raw, seed=31)
+    model = load_model(write_model(tmp_path / "m", raw, tensors), dtype=dtype)
+    oracle = plain.PlainNarurax(raw, tensors)
+    tokens = random_tokens(900, raw["vocab"], seed=14)
+    want = oracle.forward(tokens)
+    for key, off in (("size", 1), ("keep_first", -1)):          # (controls: also far keys and the last kept token matter)
+        other = copy.deepcopy(raw)
+        for layer in other["layers"]:
+            layer["mixer"]["mask"][key] += off
+        assert rel_err(plain.PlainNarurax(other, tensors).forward(tokens)[750:], want[750:]) > 20 * TOL["float32"], (key, off)
+    for cuts in ([880] + [1] * 20, [500, 2, 378] + [1] * 20):
+        cache = new_cache(model, 16, tokens=1024)
+        got = feed(model, cache, "r", tokens, cuts)
+        assert rel_err(got, want) < TOL[dtype], cuts[:3]
+        cache.close("r")
+        cache.audit()
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_and_prompts_of_one_and_two_tokens(models, name):
     model, oracle, raw, page, _ = models(name)
