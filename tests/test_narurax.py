@@ -6,7 +6,6 @@ formulation)."""
 from __future__ import annotations
 
 import copy
-import json
 import math
 
 import pytest

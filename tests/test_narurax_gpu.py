@@ -29,7 +29,6 @@ from plain import narurax_plain as plain
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
-F64 = torch.float64
 
 # Bounds on max |engine - plain| / max |plain logit| over a request, some three times the largest error
 # measured on the MI355X on these weights.
@@ -94,10 +93,6 @@ def step_meta(lengths, starts, slots):
 def close(got, want, dtype, scale=1.0):
     tol = 1e-5 if dtype == torch.float32 else 1.6e-2
     return float((got.double().cpu() - want).abs().max()) <= tol * max(scale, float(want.abs().max()))
-
-
-def dev32(t):
-    return t.to(torch.float32).cuda().contiguous()
 
 
 # ---------------------------------------------------------------------------
