@@ -6,8 +6,8 @@ as the feed-forward.
   ``(prev * mul_prev + cur * mul_cur) mod buckets``; a request's first token takes the table's last row.
 * a layer: ``x += mixer(shift(norm1(x)))``, then ``x += ff(norm2(x))``; ``shift`` moves every element
   of the normed row towards the same element of the token before by a learned share (``l<i>.shift``).
-* ``attention``: grouped heads, no biases, no value projection (the values are the keys as projected,
-  before rotation), rotation of neighbouring pairs, a sliding window that keeps the first tokens, a
+* ``attention``: grouped heads, no biases, unrotated keys that double as the values (there is no value
+  projection), rotation of neighbouring pairs, a sliding window that keeps the first tokens, a
   learned sink a head in the softmax, the heads' weights mixed after the softmax, a sigmoid gate on
   the heads' outputs.
 * ``attention_2``: biased projections, a root-mean-square norm a head on queries and keys with one

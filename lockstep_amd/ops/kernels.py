@@ -1116,7 +1116,7 @@ class Kernels:
         first, the lower index wins a tie) into ``expert [T, top]``, the softmax over the chosen logits into
         ``weight [T, top]``; the pairs ``token * top + choice`` sorted by expert into ``order``, and every
         expert's pairs cut into ``tiles [capacity, 4]`` (expert or -1, first place in ``order``, rows, 0).
-        ``scoring = "sigmoid"``: every chosen expert weighs the sigmoid of its own logit instead, not renormalised."""
+        ``scoring = "sigmoid"``: every chosen expert weighs the sigmoid of its own logit instead (the weights of a token need not add up to one)."""
         _rows_ok(logits, "experts_route logits")
         if scoring not in ("softmax", "sigmoid"):
             raise KernelError(f"experts_route: scoring is softmax or sigmoid, got {scoring!r}")

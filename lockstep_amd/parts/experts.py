@@ -6,7 +6,7 @@ that every token uses.
     w[t, k]   = softmax over the chosen logits alone
     out[t]    = sum_k w[t, k] * expert_chosen(t)[k](x[t])  +  shared(x[t])
 
-With ``score = "sigmoid"`` the weights are the chosen experts' own scores ``sigmoid(z)`` instead, not renormalised
+With ``score = "sigmoid"`` a chosen expert weighs ``sigmoid(z)`` of its own logit instead, and a token's weights need not add up to one
 (the experts with the largest scores are those with the largest logits).  With ``weigh = "input"`` a weight
 multiplies what its expert reads and not what it returns: ``out[t] = sum_k expert_chosen(t)[k](w[t, k] x[t])``.
 

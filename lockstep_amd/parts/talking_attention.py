@@ -23,9 +23,9 @@ With ``mix = "weights"`` the heads exchange their weights after each head's own 
     p_g[i, j]   = exp(raw_g[i, j]) / (exp(sink_g) + sum_j' exp(raw_g[i, j']))   (visible j'; the sink is optional)
     o_h[i]      = sigmoid(gate_h[i]) * sum_j (sum_g talk[h, g] p_g[i, j]) v_kv(h)[j]    (the gate is optional)
 
-A head's mixed weights are applied to the values of its own key/value head.  The sink has no key and no
-value and is not mixed.  This form may also have ``shared_kv`` (no value projection: the values are the
-keys as projected, before rotation) and rotates neighbouring pairs where the position encoding says so;
+A head's mixed weights are applied to the values of its own key/value head.  The sink is a bare score in a head's
+denominator: nothing is read for it and it takes no part in the mixing.  This form may also have ``shared_kv`` (the
+unrotated keys double as the values, and there is no tensor ``v``) and rotates neighbouring pairs where the position encoding says so;
 its pass in front of the attention is the one that the attention with a sink uses.  The keys are walked
 twice (statistics, then weights), because a mixed weight needs every head's finished sum.
 """

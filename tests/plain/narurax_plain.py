@@ -152,7 +152,7 @@ class PlainNarurax:
         return rotate_neighbours(q, positions, f), rotate_neighbours(k, positions, f)
 
     def attention(self, i, m, h, positions):
-        """The values are the keys before rotation; a learned sink; weights mixed over the heads; a gate."""
+        """v is k as it stood ahead of the rotation; a learned sink; weights mixed over the heads; a gate."""
         p = f"l{i}.mix"
         H, G, d = m["heads"], m["kv_heads"], m["dim"]
         n = h.shape[0]
